@@ -39,7 +39,7 @@ group can be read by another layer (`readers`): what is shared are keys and valu
 """
 from __future__ import annotations
 
-from dataclasses import dataclass
+from dataclasses import dataclass, field
 from typing import Dict, List, Optional, Sequence, Tuple
 
 import torch
@@ -56,6 +56,7 @@ class LayerCacheView:
     v_pages: Optional[torch.Tensor] = None
     block_table: Optional[torch.Tensor] = None    # int32 [B, pages per sequence], this step's sequences
     state: Optional[torch.Tensor] = None          # [slots, *shape]; index with ctx.slots
+    states: Dict[str, torch.Tensor] = field(default_factory=dict)     # the same by the request's name, for a layer with several
 
 
 class PagedGroup:
@@ -88,18 +89,20 @@ class KvGroup(PagedGroup):
         super().__init__(request, layers, n_pages)
         shape = (len(self.layers), n_pages + 1, request.heads, PAGE_SIZE, request.head_dim)
         self.k = torch.empty(shape, dtype=dtype, device=device)
-        self.v = torch.empty(shape, dtype=dtype, device=device)
+        # one vector per token that is key and value at once: the values are the keys' pages
+        self.v = torch.empty(shape, dtype=dtype, device=device) if request.values else self.k
 
     @staticmethod
     def bytes_per_token(request: CacheRequest, n_layers: int, dtype: torch.dtype) -> int:
-        return 2 * n_layers * request.heads * request.head_dim * torch.empty((), dtype=dtype).element_size()
+        sets = 2 if request.values else 1
+        return sets * n_layers * request.heads * request.head_dim * torch.empty((), dtype=dtype).element_size()
 
     def fill_view(self, view: "LayerCacheView", i: int, block_tables: Dict[int, torch.Tensor]) -> None:
         view.k_pages, view.v_pages = self.k[i], self.v[i]
         view.block_table = block_tables[id(self)]
 
     def bytes(self) -> int:
-        return 2 * self.k.numel() * self.k.element_size()
+        return (2 if self.request.values else 1) * self.k.numel() * self.k.element_size()
 
 
 class StateGroup:
@@ -125,6 +128,7 @@ class StateGroup:
 
     def fill_view(self, view: "LayerCacheView", i: int, block_tables: Dict[int, torch.Tensor]) -> None:
         view.state = self.data[i]
+        view.states[self.request.name] = self.data[i]
 
     def bytes(self) -> int:
         return self.data.numel() * self.data.element_size()
@@ -138,12 +142,21 @@ def register_cache_kind(kind: str, group_class: type) -> None:
     _GROUP_KINDS[kind] = group_class
 
 
-def bytes_per_token(requests: Sequence[Optional[CacheRequest]], dtype: torch.dtype) -> int:
+def requests_of(entry) -> List[CacheRequest]:
+    """What one layer asks for, as a list: nothing, one request, or several."""
+    if entry is None:
+        return []
+    if isinstance(entry, CacheRequest):
+        return [entry]
+    return [r for r in entry if r is not None]
+
+
+def bytes_per_token(requests: Sequence, dtype: torch.dtype) -> int:
     """Bytes that one more token of one sequence adds over all layers."""
     counts: Dict[Tuple, int] = {}
     reqs: Dict[Tuple, CacheRequest] = {}
-    for r in requests:
-        if r is not None and r.kind in _GROUP_KINDS:
+    for r in (r for entry in requests for r in requests_of(entry)):
+        if r.kind in _GROUP_KINDS:
             counts[r.key()] = counts.get(r.key(), 0) + 1
             reqs[r.key()] = r
     return sum(_GROUP_KINDS[reqs[k].kind].bytes_per_token(reqs[k], n, dtype) for k, n in counts.items())
@@ -152,7 +165,8 @@ def bytes_per_token(requests: Sequence[Optional[CacheRequest]], dtype: torch.dty
 class Cache:
     def __init__(self, requests: Sequence[Optional[CacheRequest]], n_slots: int, max_tokens: int,
                  dtype: torch.dtype, device, readers: Optional[Dict[int, int]] = None):
-        """requests[l]: what the mixer at place l of the schedule asked for (None: nothing);
+        """requests[l]: what the layer at place l of the schedule asked for (None: nothing; one request, or a
+        list of requests with different names);
         "layer" below means such a place.  readers[l] = j: place l reads place j's keys and
         values.  max_tokens: positions the pages of each
         group hold together, every sequence rounded up to whole pages."""
@@ -169,14 +183,17 @@ class Cache:
         self.layer_groups: Dict[int, List[Tuple[object, int]]] = {}
         by_key: Dict[Tuple, List[int]] = {}
         reqs: Dict[Tuple, CacheRequest] = {}
-        for l, r in enumerate(requests):
-            if r is None:
-                continue
-            if r.kind not in _GROUP_KINDS:
-                raise CacheError(f"layer {l} asks for an unknown kind of cache {r.kind!r} "
-                                 f"(known: {', '.join(sorted(_GROUP_KINDS))})")
-            by_key.setdefault(r.key(), []).append(l)
-            reqs[r.key()] = r
+        for l, entry in enumerate(requests):
+            seen = set()
+            for r in requests_of(entry):
+                if r.kind not in _GROUP_KINDS:
+                    raise CacheError(f"layer {l} asks for an unknown kind of cache {r.kind!r} "
+                                     f"(known: {', '.join(sorted(_GROUP_KINDS))})")
+                if r.key() in seen:
+                    raise CacheError(f"layer {l} asks twice for the same thing (give its requests different names)")
+                seen.add(r.key())
+                by_key.setdefault(r.key(), []).append(l)
+                reqs[r.key()] = r
         for key, layers in by_key.items():
             r = reqs[key]
             g = _GROUP_KINDS[r.kind](r, layers, self.n_pages, self.n_slots, dtype, device)

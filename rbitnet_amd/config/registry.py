@@ -6,8 +6,9 @@ keys whatever `general.architecture` says (gguf/bitnet_meta.rs:27-28) and uses
 the name only as a label (gguf/parse.rs:222-234).
 
 A configuration class has: `from_dict(dict)`, `to_dict()`, `to_spec()` and
-optionally `tensor_aliases(name) -> [alternate names]` and `with_tensor_names(names)
--> configuration` (what the names in a weight file decide where config.json is silent).
+optionally `tensor_aliases(name) -> [alternate names]`, `with_tensor_names(names)
+-> configuration` (what the names in a weight file decide where config.json is silent) and
+`with_tensor_shapes({name: shape}) -> configuration` (sizes that only the weight file holds).
 """
 from __future__ import annotations
 
@@ -16,6 +17,7 @@ import os
 from typing import Any, Dict, Iterable, Optional, Tuple
 
 from ..errors import ConfigError
+from .bagonex import BagonexConfig
 from .llama import LlamaConfig
 from .spec import ModelSpec
 
@@ -38,7 +40,7 @@ def config_class_for(name: str) -> Any:
 
 
 def architecture_of(config: Dict[str, Any]) -> str:
-    archs = config.get("architectures")
+    archs = config.get("architectures", config.get("architecture"))
     if isinstance(archs, list) and archs:
         return str(archs[0])
     if isinstance(archs, str):
@@ -50,9 +52,11 @@ def architecture_of(config: Dict[str, Any]) -> str:
     raise ConfigError("config.json names no architecture (key 'architectures')")
 
 
-def load_config(path_or_dict: Any, tensor_names: Optional[Iterable[str]] = None) -> Tuple[Any, ModelSpec]:
+def load_config(path_or_dict: Any, tensor_names: Optional[Iterable[str]] = None,
+                tensor_shapes: Optional[Dict[str, Any]] = None) -> Tuple[Any, ModelSpec]:
     """config.json (a folder, a file or an already parsed dict) -> (typed
-    configuration, spec).  tensor_names: the names in the weight file that goes with it."""
+    configuration, spec).  tensor_names: the names in the weight file that goes with it;
+    tensor_shapes: name -> shape of the same, for a configuration that reads sizes off them."""
     if isinstance(path_or_dict, dict):
         raw = path_or_dict
     else:
@@ -72,7 +76,10 @@ def load_config(path_or_dict: Any, tensor_names: Optional[Iterable[str]] = None)
     cfg = cls.from_dict(raw)
     if tensor_names is not None and hasattr(cfg, "with_tensor_names"):
         cfg = cfg.with_tensor_names(list(tensor_names))
+    if tensor_shapes is not None and hasattr(cfg, "with_tensor_shapes"):
+        cfg = cfg.with_tensor_shapes(tensor_shapes)
     return cfg, cfg.to_spec()
 
 
 register_architecture("LlamaForCausalLM", LlamaConfig)
+register_architecture("Bagonex", BagonexConfig)

@@ -42,11 +42,13 @@ class LayerSpec:
     prefix: str
     block: str
     mixer: PartSpec
-    feed_forward: PartSpec
+    feed_forward: Optional[PartSpec]          # None: the layer has no feed-forward (for arrangements that allow it)
     norm1: PartSpec
-    norm2: PartSpec
+    norm2: Optional[PartSpec]
     # tensor-name segment of each part below `prefix`, e.g. {"mixer": "self_attn"}
     segments: Optional[Dict[str, str]] = None
+    # what the arrangement itself takes (copies of the stream, a convolution in front of the mixer, ...)
+    params: Dict[str, Any] = field(default_factory=dict)
 
 
 @dataclass

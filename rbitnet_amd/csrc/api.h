@@ -117,6 +117,68 @@ int rb_attention_decode_fused_bf16(const float* qkv, int qkv_terms, long long qk
                                    int bt_stride, int n_seqs, int n_heads, int n_kv_heads, int head_dim, float scale,
                                    int window, int n_splits, float* workspace, void* stream);
 
+// rb_attention_generic with a sink per query head (sinks float32 [Hq], null: none): the softmax's denominator also
+// holds exp(sink), a score that is not scaled and has no key and no value.  v_pages may be k_pages (attention over
+// cached latents, which are keys and values at once).
+int rb_attention_generic_sinks(const void* q, const void* k_pages, const void* v_pages, void* out, int dtype,
+                               const int32_t* tok_pos, const int32_t* tok_seq, const int32_t* block_table,
+                               int bt_stride, int n_tokens, int n_heads, int n_kv_heads, int head_dim, float scale,
+                               int window, const float* sinks, void* stream);
+
+// ---- a residual stream in several copies, layer norm, xIELU, the cap of logits (streams.hip)
+// x [S, T, E] float32, stream_stride floats from one copy to the next.
+//   rb_embed_streams:     x[s][t, :] = table[ids[t], :] for every copy
+//   rb_streams_layernorm: u = sum_s coef[s] x[s][src] (+ delta[src]), src = rows ? rows[r] : r;
+//                         out[r] = (u - mean) / sqrt(var + eps) * weight + bias (variance: mean of squared deviations).
+//                         coef null: all 1; bias null: none; one stream with a delta and no rows: x = u as well.
+//   rb_streams_update:    x'[j] = sum_s mix[s * S + j] x[s] + out_coef[j] * (scale ? scale[e] : 1) * y, all copies at once
+int rb_embed_streams(const void* table, int table_dtype, const int32_t* ids, float* x, int n_streams, long long stream_stride,
+                     int n_tokens, int width, void* stream);
+int rb_streams_layernorm(float* x, int n_streams, long long stream_stride, const float* coef, const float* delta,
+                         const float* weight, const float* bias, float eps, const int32_t* rows, int n_rows, int width,
+                         void* out, int out_dtype, void* stream);
+int rb_streams_update(float* x, int n_streams, long long stream_stride, const float* mix, const float* out_coef, const float* y,
+                      const float* scale, int n_tokens, int width, void* stream);
+// out = z > 0 ? softplus(act[0]) z^2 + z/2 : (1/2 + softplus(act[1])) (exp(z) - 1 - z) + z/2
+int rb_xielu(const float* z, const float* act, void* out, int out_dtype, long long n, void* stream);
+// x <- cap * tanh(x / cap)
+int rb_tanh_cap(float* x, float cap, long long n, void* stream);
+
+// ---- layers with a fixed-size state per sequence (recurrent.hip)
+// Causal convolution over time per channel: y[t, c] = (residual ? x[t, c] : 0) + sum_d w[c, taps-1-d] x[t-d, c], act 1: silu.
+// x float32 rows x_stride apart; rows before the step come from state [slots, taps-1, C] (the sequence's last taps-1
+// inputs, oldest first; zero for a fresh slot).  rb_short_conv_state, afterwards, moves the state on by the step's rows.
+int rb_short_conv(const float* x, long long x_stride, const float* w, int taps, const float* state, const int32_t* tok_pos,
+                  const int32_t* tok_seq, const int32_t* past_len, const int32_t* slots, void* out, long long out_stride,
+                  int out_dtype, int residual, int act, int n_tokens, int channels, void* stream);
+int rb_short_conv_state(const float* x, long long x_stride, int taps, float* state, const int32_t* cu_seqlens,
+                        const int32_t* slots, int n_seqs, int channels, void* stream);
+// What enters the gated delta rule, in place: qk [T, qk_stride] holds Hk q heads, then Hk k heads, of `dim` numbers;
+// each becomes x / sqrt(sum x^2 + unit_eps), q times q_scale.  a [T, H, dim] (rows a_stride apart) becomes the decay
+// exp(-exp(a_log[h]) softplus(a + dt_bias)); beta [T, H] = sigmoid(b_in[t * b_stride + h]).
+int rb_delta_prep(float* qk, long long qk_stride, int n_kv_heads, int dim, float* a, long long a_stride, const float* dt_bias, const float* a_log,
+                  int n_heads, const float* b_in, long long b_stride, float* beta, float q_scale, float unit_eps, int n_tokens,
+                  void* stream);
+// Per sequence b (rows cu_seqlens[b]..) and head h, token after token on state [slots, H, dim, vdim]:
+//   S <- diag(g) S;  u = beta (v - S^T k);  S <- S + k u^T;  out[t, h, :] = S^T q      (head h reads q/k head h / (H / Hk))
+int rb_delta_rule(const float* q, const float* k, long long qk_stride, const float* v, long long v_stride, const float* g,
+                  long long g_stride, const float* beta, float* state, const int32_t* cu_seqlens, const int32_t* slots, float* out, int n_seqs,
+                  int n_heads, int n_kv_heads, int dim, int vdim, void* stream);
+// out[t, h, :] = o / sqrt(mean(o^2) + eps) * weight[vdim] * sigmoid(gate[t * gate_stride + h * vdim + :])
+int rb_gated_rmsnorm(const float* o, const float* weight, const float* gate, long long gate_stride, float eps, void* out,
+                     int out_dtype, int n_tokens, int n_heads, int vdim, void* stream);
+
+// ---- attention through a latent (latent.hip)
+// Per token: cq = rmsnorm(proj[t, 0:q_rank]) * q_gain -> cq [T, q_rank]; rmsnorm(proj[t, kv_col:+kv_rank]) * kv_gain ->
+// the token's place in pages [n_pages, 1, 64, kv_rank].  A rank of 0 leaves that half out.
+int rb_latent_norm_store(const float* proj, long long stride, int q_rank, const float* q_gain, void* cq, int kv_col,
+                         int kv_rank, const float* kv_gain, void* pages, int dtype, const int32_t* tok_pos,
+                         const int32_t* tok_seq, const int32_t* block_table, int bt_stride, float eps, int n_tokens,
+                         void* stream);
+// y[t, h, n] = sum_k w[h, k, n] x[t, h, k]
+int rb_heads_linear(const void* x, int x_dtype, const void* w, int w_dtype, void* y, int y_dtype, int n_tokens, int n_heads,
+                    int n, int k, void* stream);
+
 // tokens[r] = argmax of logits[r, :] (NaN counts as -inf, lowest index among equals), or, where
 // temperature[r] > 0, the first index whose running sum of exp(z/T - max) reaches u[r] times the total.
 // workspace: rb_sample_workspace_bytes(n_rows, vocab) bytes, 8-byte aligned, contents do not matter.

@@ -24,7 +24,7 @@ __global__ __launch_bounds__(RB_WAVE * AG_MAX_WAVES) void attention_generic_kern
     const T* __restrict__ q, const T* __restrict__ k_pages, const T* __restrict__ v_pages, T* __restrict__ out,
     const int32_t* __restrict__ tok_pos, const int32_t* __restrict__ tok_seq,
     const int32_t* __restrict__ block_table, int bt_stride, int n_heads, int n_kv, int head_dim, float scale,
-    int window) {
+    int window, const float* __restrict__ sinks) {
   __shared__ float qs[AG_MAX_D];
   __shared__ float ps_all[AG_MAX_WAVES][RB_PAGE];
   __shared__ float red_m[AG_MAX_WAVES], red_l[AG_MAX_WAVES];
@@ -94,6 +94,7 @@ __global__ __launch_bounds__(RB_WAVE * AG_MAX_WAVES) void attention_generic_kern
     if (wave != 0) return;
     float mx = red_m[0];
     for (int w = 1; w < n_waves; ++w) mx = fmaxf(mx, red_m[w]);
+    m_run = mx;
     l_run = 0.f;
 #pragma unroll
     for (int i = 0; i < AG_MAX_D / RB_WAVE; ++i) acc[i] = 0.f;
@@ -107,6 +108,7 @@ __global__ __launch_bounds__(RB_WAVE * AG_MAX_WAVES) void attention_generic_kern
       }
     }
   }
+  if (sinks) l_run += expf(sinks[h] - m_run);          // a term of the denominator with no key and no value
   const float inv = l_run > 0.f ? 1.0f / l_run : 0.f;
   T* orow = out + ((size_t)t * n_heads + h) * head_dim;
 #pragma unroll
@@ -143,7 +145,7 @@ __global__ __launch_bounds__(RB_WAVE * AG_MAX_WAVES) void attention_generic_vec_
     const T* __restrict__ q, const T* __restrict__ k_pages, const T* __restrict__ v_pages, T* __restrict__ out,
     const int32_t* __restrict__ tok_pos, const int32_t* __restrict__ tok_seq,
     const int32_t* __restrict__ block_table, int bt_stride, int n_heads, int n_kv, int head_dim, float scale,
-    int window, int group_lanes) {
+    int window, int group_lanes, const float* __restrict__ sinks) {
   __shared__ __attribute__((aligned(16))) float qs[AG_MAX_D];
   __shared__ float ps_all[AG_MAX_WAVES][RB_PAGE];
   __shared__ float red_m[AG_MAX_WAVES], red_l[AG_MAX_WAVES];
@@ -228,6 +230,7 @@ __global__ __launch_bounds__(RB_WAVE * AG_MAX_WAVES) void attention_generic_vec_
     if (wave != 0) return;
     float mx = red_m[0];
     for (int w = 1; w < n_waves; ++w) mx = fmaxf(mx, red_m[w]);
+    m_run = mx;
     l_run = 0.f;
     acc = make_float4(0.f, 0.f, 0.f, 0.f);
     for (int w = 0; w < n_waves; ++w) {
@@ -243,6 +246,7 @@ __global__ __launch_bounds__(RB_WAVE * AG_MAX_WAVES) void attention_generic_vec_
     }
   }
   if (owner) {
+    if (sinks) l_run += expf(sinks[h] - m_run);        // a term of the denominator with no key and no value
     const float inv = l_run > 0.f ? 1.0f / l_run : 0.f;
     T* orow = out + ((size_t)t * n_heads + h) * head_dim + 4 * c;
     Num<T>::store(orow + 0, acc.x * inv);
@@ -259,8 +263,18 @@ extern "C" int rb_attention_generic(const void* q, const void* k_pages, const vo
                                     const int32_t* tok_pos, const int32_t* tok_seq, const int32_t* block_table,
                                     int bt_stride, int n_tokens, int n_heads, int n_kv_heads, int head_dim,
                                     float scale, int window, void* stream) {
-  RB_RECORDED(rb_attention_generic(q, k_pages, v_pages, out, dtype, tok_pos, tok_seq, block_table, bt_stride, n_tokens, n_heads,
-                                   n_kv_heads, head_dim, scale, window, stream));
+  return rb_attention_generic_sinks(q, k_pages, v_pages, out, dtype, tok_pos, tok_seq, block_table, bt_stride, n_tokens,
+                                    n_heads, n_kv_heads, head_dim, scale, window, nullptr, stream);
+}
+
+// The same with a sink per query head (sinks float32 [Hq], null: none): the softmax's denominator also holds
+// exp(sink), a score that is not scaled and belongs to no key and no value.  v_pages may be k_pages.
+extern "C" int rb_attention_generic_sinks(const void* q, const void* k_pages, const void* v_pages, void* out, int dtype,
+                                          const int32_t* tok_pos, const int32_t* tok_seq, const int32_t* block_table,
+                                          int bt_stride, int n_tokens, int n_heads, int n_kv_heads, int head_dim,
+                                          float scale, int window, const float* sinks, void* stream) {
+  RB_RECORDED(rb_attention_generic_sinks(q, k_pages, v_pages, out, dtype, tok_pos, tok_seq, block_table, bt_stride, n_tokens,
+                                         n_heads, n_kv_heads, head_dim, scale, window, sinks, stream));
   RB_REQUIRE(n_tokens >= 0 && n_heads > 0 && n_kv_heads > 0 && n_heads % n_kv_heads == 0,
              "rb_attention_generic: bad head counts Hq=%d Hk=%d", n_heads, n_kv_heads);
   RB_REQUIRE(head_dim > 0 && head_dim % 2 == 0 && head_dim <= AG_MAX_D,
@@ -282,12 +296,12 @@ extern "C" int rb_attention_generic(const void* q, const void* k_pages, const vo
       attention_generic_vec_kernel<float><<<grid, threads, 0, s>>>((const float*)q, (const float*)k_pages,
                                                                   (const float*)v_pages, (float*)out, tok_pos, tok_seq,
                                                                   block_table, bt_stride, n_heads, n_kv_heads, head_dim,
-                                                                  scale, window, group_lanes);
+                                                                  scale, window, group_lanes, sinks);
     else
       attention_generic_vec_kernel<bf16_t><<<grid, threads, 0, s>>>((const bf16_t*)q, (const bf16_t*)k_pages,
                                                                    (const bf16_t*)v_pages, (bf16_t*)out, tok_pos,
                                                                    tok_seq, block_table, bt_stride, n_heads, n_kv_heads,
-                                                                   head_dim, scale, window, group_lanes);
+                                                                   head_dim, scale, window, group_lanes, sinks);
     RB_LAUNCH_CHECK();
     return 0;
   }
@@ -295,12 +309,12 @@ extern "C" int rb_attention_generic(const void* q, const void* k_pages, const vo
     attention_generic_kernel<float><<<grid, threads, 0, s>>>((const float*)q, (const float*)k_pages,
                                                             (const float*)v_pages, (float*)out, tok_pos, tok_seq,
                                                             block_table, bt_stride, n_heads, n_kv_heads, head_dim,
-                                                            scale, window);
+                                                            scale, window, sinks);
   else if (dtype == RB_BF16)
     attention_generic_kernel<bf16_t><<<grid, threads, 0, s>>>((const bf16_t*)q, (const bf16_t*)k_pages,
                                                              (const bf16_t*)v_pages, (bf16_t*)out, tok_pos,
                                                              tok_seq, block_table, bt_stride, n_heads, n_kv_heads,
-                                                             head_dim, scale, window);
+                                                             head_dim, scale, window, sinks);
   else
     RB_REQUIRE(false, "rb_attention_generic: unknown dtype %d", dtype);
   RB_LAUNCH_CHECK();

@@ -20,6 +20,7 @@ _F32, _BF16 = 0, 1
 _P = ctypes.c_void_p
 _I = ctypes.c_int
 _F = ctypes.c_float
+_L = ctypes.c_longlong
 
 
 def dtype_code(dtype: torch.dtype) -> int:
@@ -104,7 +105,8 @@ class KernelTimes:
         return "\n".join(lines)
 
 
-TIMED_OPS = ("embed_gather", "add_rmsnorm", "rope_kv_write", "swiglu", "gemm_generic", "gemm_bf16", "gemm_bf16_terms",
+TIMED_OPS = ("embed_streams", "streams_layernorm", "streams_update", "xielu", "tanh_cap", "short_conv", "short_conv_state",
+             "delta_prep", "delta_rule", "gated_rmsnorm", "latent_norm_store", "heads_linear", "embed_gather", "add_rmsnorm", "rope_kv_write", "swiglu", "gemm_generic", "gemm_bf16", "gemm_bf16_terms",
              "gemm_bf16_few", "attention_generic", "attention_prefill_bf16", "attention_decode_bf16",
              "attention_decode_fused_bf16", "sample")
 
@@ -145,6 +147,19 @@ class Kernels:
             "rb_place_rows": [_P, _I, _P, _I, _I] + [ctypes.c_longlong] * 6 + [_P],
             "rb_probe_read": [_P, ctypes.c_longlong, _I, _I, _P, _P],
             "rb_probe_mfma": [_I, _I, _P, _P],
+            "rb_attention_generic_sinks": [_P, _P, _P, _P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _F, _I, _P, _P],
+            "rb_embed_streams": [_P, _I, _P, _P, _I, _L, _I, _I, _P],
+            "rb_streams_layernorm": [_P, _I, _L, _P, _P, _P, _P, _F, _P, _I, _I, _P, _I, _P],
+            "rb_streams_update": [_P, _I, _L, _P, _P, _P, _P, _I, _I, _P],
+            "rb_xielu": [_P, _P, _P, _I, _L, _P],
+            "rb_tanh_cap": [_P, _F, _L, _P],
+            "rb_short_conv": [_P, _L, _P, _I, _P, _P, _P, _P, _P, _P, _L, _I, _I, _I, _I, _I, _P],
+            "rb_short_conv_state": [_P, _L, _I, _P, _P, _P, _I, _I, _P],
+            "rb_delta_prep": [_P, _L, _I, _I, _P, _L, _P, _P, _I, _P, _L, _P, _F, _F, _I, _P],
+            "rb_delta_rule": [_P, _P, _L, _P, _L, _P, _L, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _P],
+            "rb_gated_rmsnorm": [_P, _P, _P, _L, _F, _P, _I, _I, _I, _I, _P],
+            "rb_latent_norm_store": [_P, _L, _I, _P, _P, _I, _I, _P, _P, _I, _P, _P, _P, _I, _F, _I, _P],
+            "rb_heads_linear": [_P, _I, _P, _I, _P, _I, _I, _I, _I, _I, _P],
         }
         for name, args in sig.items():
             fn = getattr(L, name)
@@ -411,6 +426,207 @@ class Kernels:
             raise KernelError("sampling workspace too small")
         self._ok(self._lib.rb_sample(_ptr(logits), n, vocab, _ptr(temperature), _ptr(u), _ptr(tokens),
                                      _ptr(workspace), self._stream()))
+
+    # ------------------------------------------------------------------ streams, layer norm, activations
+    def embed_streams(self, table: torch.Tensor, ids: torch.Tensor, x: torch.Tensor) -> None:
+        """x [S, T, E] float32: every copy s gets table[ids[t]] in row t."""
+        s_, n, width = x.shape
+        _check(table, "table")
+        _check(ids, "ids", torch.int32, (n,))
+        _check(x, "x", torch.float32)
+        if table.shape[1] != width:
+            raise KernelError("embedding width mismatch")
+        self._ok(self._lib.rb_embed_streams(_ptr(table), dtype_code(table.dtype), _ptr(ids), _ptr(x), s_, n * width, n, width,
+                                            self._stream()))
+
+    def streams_layernorm(self, x: torch.Tensor, coef: Optional[torch.Tensor], weight: torch.Tensor,
+                          bias: Optional[torch.Tensor], eps: float, rows: Optional[torch.Tensor], out: torch.Tensor,
+                          delta: Optional[torch.Tensor] = None) -> None:
+        """x [S, T, E] (or [T, E]: one stream) float32; out [rows or T, E]: the layer norm of sum_s coef[s] x[s]."""
+        if x.dim() == 2:
+            x = x.unsqueeze(0)
+        s_, n, width = x.shape
+        _check(x, "x", torch.float32)
+        if coef is not None:
+            _check(coef, "coef", torch.float32, (s_,))
+        _check(weight, "weight", torch.float32, (width,))
+        if bias is not None:
+            _check(bias, "bias", torch.float32, (width,))
+        if delta is not None:
+            _check(delta, "delta", torch.float32, (n, width))
+        n_rows = n
+        if rows is not None:
+            n_rows = rows.shape[0]
+            _check(rows, "rows", torch.int32, (n_rows,))
+        _check(out, "out", None, (n_rows, width))
+        self._ok(self._lib.rb_streams_layernorm(_ptr(x), s_, n * width, _ptr(coef), _ptr(delta), _ptr(weight), _ptr(bias),
+                                                float(eps), _ptr(rows), n_rows, width, _ptr(out), dtype_code(out.dtype),
+                                                self._stream()))
+
+    def streams_update(self, x: torch.Tensor, mix: torch.Tensor, out_coef: torch.Tensor, y: torch.Tensor,
+                       scale: Optional[torch.Tensor]) -> None:
+        """x [S, T, E] <- mix^T x + out_coef (scale * y), every copy from all the old ones."""
+        s_, n, width = x.shape
+        _check(x, "x", torch.float32)
+        _check(mix, "mix", torch.float32, (s_, s_))
+        _check(out_coef, "out_coef", torch.float32, (s_,))
+        _check(y, "y", torch.float32, (n, width))
+        if scale is not None:
+            _check(scale, "scale", torch.float32, (width,))
+        self._ok(self._lib.rb_streams_update(_ptr(x), s_, n * width, _ptr(mix), _ptr(out_coef), _ptr(y), _ptr(scale), n, width,
+                                             self._stream()))
+
+    def xielu(self, z: torch.Tensor, act: torch.Tensor, out: torch.Tensor) -> None:
+        _check(z, "z", torch.float32)
+        _check(act, "act", torch.float32, (2,))
+        _check(out, "out", None, z.shape)
+        self._ok(self._lib.rb_xielu(_ptr(z), _ptr(act), _ptr(out), dtype_code(out.dtype), z.numel(), self._stream()))
+
+    def tanh_cap(self, x: torch.Tensor, cap: float) -> None:
+        _check(x, "x", torch.float32)
+        self._ok(self._lib.rb_tanh_cap(_ptr(x), float(cap), x.numel(), self._stream()))
+
+    # ------------------------------------------------------------------ layers with a state per sequence
+    def short_conv(self, x: torch.Tensor, col0: int, channels: int, w: torch.Tensor, state: Optional[torch.Tensor], ctx,
+                   out: torch.Tensor, residual: bool, act: int) -> None:
+        """Columns col0 .. col0 + channels of x [T, W] float32 through the causal convolution w [channels, taps];
+        state [slots, taps - 1, channels] float32 holds every sequence's last inputs."""
+        n, width = x.shape
+        taps = w.shape[1]
+        _check(x, "x", torch.float32)
+        _check(w, "w", torch.float32, (channels, taps))
+        if col0 < 0 or col0 + channels > width:
+            raise KernelError("short_conv: the columns lie outside the rows")
+        if taps > 1:
+            _check(state, "state", torch.float32)
+            if tuple(state.shape[1:]) != (taps - 1, channels):
+                raise KernelError(f"short_conv: state of shape {tuple(state.shape)}, expected [*, {taps - 1}, {channels}]")
+        _check(out, "out", None, (n, channels))
+        _check(ctx.tok_pos, "tok_pos", torch.int32, (n,))
+        self._ok(self._lib.rb_short_conv(x.data_ptr() + 4 * col0, width, _ptr(w), taps, _ptr(state) if taps > 1 else None,
+                                         _ptr(ctx.tok_pos), _ptr(ctx.tok_seq), _ptr(ctx.past_len), _ptr(ctx.slots), _ptr(out),
+                                         channels, dtype_code(out.dtype), int(bool(residual)), int(act), n, channels,
+                                         self._stream()))
+
+    def short_conv_state(self, x: torch.Tensor, col0: int, channels: int, taps: int, state: torch.Tensor, ctx) -> None:
+        """After `short_conv`: the state moves on by the step's rows."""
+        if taps <= 1:
+            return
+        n, width = x.shape
+        _check(x, "x", torch.float32)
+        _check(state, "state", torch.float32)
+        if tuple(state.shape[1:]) != (taps - 1, channels) or col0 < 0 or col0 + channels > width:
+            raise KernelError("short_conv_state: state or columns do not fit")
+        self._ok(self._lib.rb_short_conv_state(x.data_ptr() + 4 * col0, width, taps, _ptr(state), _ptr(ctx.cu_seqlens),
+                                               _ptr(ctx.slots), ctx.n_seqs, channels, self._stream()))
+
+    def delta_prep(self, qkv: torch.Tensor, n_kv: int, dim: int, a: torch.Tensor, dt_bias: torch.Tensor, a_log: torch.Tensor,
+                   n_heads: int, b_in: torch.Tensor, b_col: int, beta: torch.Tensor, q_scale: float, unit_eps: float) -> None:
+        """In place: the q and k heads at the start of qkv's rows become unit vectors, the first H * dim columns of a
+        the decays; beta [T, H] = sigmoid of columns b_col .. of b_in."""
+        n, width = qkv.shape
+        _check(qkv, "qkv", torch.float32)
+        if width < 2 * n_kv * dim:
+            raise KernelError("delta_prep: rows too short for the q and k heads")
+        _check(a, "a", torch.float32)
+        if a.shape[0] != n or a.shape[1] < n_heads * dim:
+            raise KernelError("delta_prep: rows of a too short for the decays")
+        _check(dt_bias, "dt_bias", torch.float32, (n_heads * dim,))
+        _check(a_log, "a_log", torch.float32, (n_heads,))
+        _check(b_in, "b_in", torch.float32)
+        if b_in.shape[0] != n or b_col < 0 or b_col + n_heads > b_in.shape[1]:
+            raise KernelError("delta_prep: the beta columns lie outside the rows")
+        _check(beta, "beta", torch.float32, (n, n_heads))
+        self._ok(self._lib.rb_delta_prep(_ptr(qkv), width, n_kv, dim, _ptr(a), a.shape[1], _ptr(dt_bias), _ptr(a_log), n_heads,
+                                         b_in.data_ptr() + 4 * b_col, b_in.shape[1], _ptr(beta), float(q_scale), float(unit_eps),
+                                         n, self._stream()))
+
+    def delta_rule(self, qkv: torch.Tensor, n_kv: int, dim: int, n_heads: int, vdim: int, g: torch.Tensor,
+                   beta: torch.Tensor, state: torch.Tensor, ctx, out: torch.Tensor) -> None:
+        """qkv [T, >= (2 Hk dim + H vdim)] float32: q heads, k heads, v heads; state [slots, H, dim, vdim] float32."""
+        n, width = qkv.shape
+        _check(qkv, "qkv", torch.float32)
+        if width < 2 * n_kv * dim + n_heads * vdim:
+            raise KernelError("delta_rule: rows too short for q, k and v")
+        _check(g, "g", torch.float32)
+        if g.shape[0] != n or g.shape[1] < n_heads * dim:
+            raise KernelError("delta_rule: rows of g too short for the decays")
+        _check(beta, "beta", torch.float32, (n, n_heads))
+        _check(state, "state", torch.float32)
+        if tuple(state.shape[1:]) != (n_heads, dim, vdim):
+            raise KernelError(f"delta_rule: state of shape {tuple(state.shape)}, expected [*, {n_heads}, {dim}, {vdim}]")
+        _check(out, "out", torch.float32, (n, n_heads * vdim))
+        if ctx.n_tokens != n:
+            raise KernelError("delta_rule: the step's tokens and the rows differ")
+        base = qkv.data_ptr()
+        self._ok(self._lib.rb_delta_rule(base, base + 4 * n_kv * dim, width, base + 8 * n_kv * dim, width, _ptr(g), g.shape[1], _ptr(beta),
+                                         _ptr(state), _ptr(ctx.cu_seqlens), _ptr(ctx.slots), _ptr(out), ctx.n_seqs, n_heads,
+                                         n_kv, dim, vdim, self._stream()))
+
+    def gated_rmsnorm(self, o: torch.Tensor, weight: torch.Tensor, gate: torch.Tensor, gate_col: int, eps: float,
+                      n_heads: int, vdim: int, out: torch.Tensor) -> None:
+        n = o.shape[0]
+        _check(o, "o", torch.float32, (n, n_heads * vdim))
+        _check(weight, "weight", torch.float32, (vdim,))
+        _check(gate, "gate", torch.float32)
+        if gate.shape[0] != n or gate_col < 0 or gate_col + n_heads * vdim > gate.shape[1]:
+            raise KernelError("gated_rmsnorm: the gate's columns lie outside the rows")
+        _check(out, "out", None, (n, n_heads * vdim))
+        self._ok(self._lib.rb_gated_rmsnorm(_ptr(o), _ptr(weight), gate.data_ptr() + 4 * gate_col, gate.shape[1], float(eps),
+                                            _ptr(out), dtype_code(out.dtype), n, n_heads, vdim, self._stream()))
+
+    # ------------------------------------------------------------------ attention through a latent
+    def latent_norm_store(self, proj: torch.Tensor, q_rank: int, q_gain: Optional[torch.Tensor], cq: Optional[torch.Tensor],
+                          kv_rank: int, kv_gain: Optional[torch.Tensor], pages: Optional[torch.Tensor], ctx, block_table,
+                          eps: float, dtype: torch.dtype) -> None:
+        """proj [T, q_rank + kv_rank] float32: the two down-projections; cq [T, q_rank] and the pages
+        [*, 1, 64, kv_rank] get their RMS norms (kv_rank 0: no latent is stored)."""
+        n, width = proj.shape
+        _check(proj, "proj", torch.float32, (n, q_rank + kv_rank))
+        if q_rank:
+            _check(q_gain, "q_gain", torch.float32, (q_rank,))
+            _check(cq, "cq", dtype, (n, q_rank))
+        if kv_rank:
+            _check(kv_gain, "kv_gain", torch.float32, (kv_rank,))
+            _check(pages, "pages", dtype)
+            if tuple(pages.shape[1:]) != (1, self.page_size, kv_rank):
+                raise KernelError(f"latent pages have shape {tuple(pages.shape)}, expected [*, 1, {self.page_size}, {kv_rank}]")
+            _check(block_table, "block_table", torch.int32)
+        self._ok(self._lib.rb_latent_norm_store(_ptr(proj), width, q_rank, _ptr(q_gain), _ptr(cq), q_rank, kv_rank, _ptr(kv_gain),
+                                                _ptr(pages) if kv_rank else None, dtype_code(dtype), _ptr(ctx.tok_pos),
+                                                _ptr(ctx.tok_seq), _ptr(block_table) if kv_rank else None,
+                                                block_table.shape[1] if kv_rank else 0, float(eps), n, self._stream()))
+
+    def heads_linear(self, x: torch.Tensor, w: torch.Tensor, y: torch.Tensor) -> None:
+        """y[t, h, :] = w[h]^T x[t, h, :] with w [H, K, N]; x [T, H * K], y [T, H * N]."""
+        h, k, n_out = w.shape
+        n = x.shape[0]
+        _check(x, "x", None, (n, h * k))
+        _check(w, "w")
+        _check(y, "y", None, (n, h * n_out))
+        self._ok(self._lib.rb_heads_linear(_ptr(x), dtype_code(x.dtype), _ptr(w), dtype_code(w.dtype), _ptr(y),
+                                           dtype_code(y.dtype), n, h, n_out, k, self._stream()))
+
+    def attention_sinks(self, q, k_pages, v_pages, out, tok_pos, tok_seq, block_table, n_heads, n_kv, head_dim,
+                        scale, window, sinks) -> None:
+        """`attention_generic` with a sink per query head in the softmax's denominator (sinks float32 [Hq] or None);
+        v_pages may be k_pages itself."""
+        n = q.shape[0]
+        _check(q, "q", None, (n, n_heads, head_dim))
+        _check(k_pages, "k_pages", q.dtype)
+        _check(v_pages, "v_pages", q.dtype, k_pages.shape)
+        if tuple(k_pages.shape[1:]) != (n_kv, self.page_size, head_dim):
+            raise KernelError("cache pages do not match the head counts")
+        _check(out, "out", q.dtype, (n, n_heads * head_dim))
+        _check(tok_pos, "tok_pos", torch.int32, (n,))
+        _check(tok_seq, "tok_seq", torch.int32, (n,))
+        _check(block_table, "block_table", torch.int32)
+        if sinks is not None:
+            _check(sinks, "sinks", torch.float32, (n_heads,))
+        self._ok(self._lib.rb_attention_generic_sinks(_ptr(q), _ptr(k_pages), _ptr(v_pages), _ptr(out), dtype_code(q.dtype),
+                                                      _ptr(tok_pos), _ptr(tok_seq), _ptr(block_table), block_table.shape[1],
+                                                      n, n_heads, n_kv, head_dim, float(scale), int(window or 0),
+                                                      _ptr(sinks), self._stream()))
 
     # ------------------------------------------------------------------ recorded steps
     def plan_begin(self) -> int:

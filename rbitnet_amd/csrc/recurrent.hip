@@ -1,0 +1,306 @@
+// Layers that carry a fixed-size state from token to token: the short causal convolution over time
+// (per channel, a few taps) and the gated delta rule (per head a matrix S [key dim, value dim] that
+// decays per key channel, is corrected towards the new value along the new key, and is read with the
+// query).  States are float32 and live in the cache's per-slot storage; a step brings any number of
+// tokens per sequence on top of what the state holds.  All arithmetic here is float32.
+#include <math.h>
+
+#include "api.h"
+#include "common.h"
+
+__device__ __forceinline__ float rb_sigmoid(float v) { return 1.0f / (1.0f + expf(-v)); }
+__device__ __forceinline__ float rb_softplus(float v) { return v > 20.0f ? v : log1pf(expf(v)); }
+
+// ---------------------------------------------------------------- short convolution
+// y[t, c] = (residual ? x[t, c] : 0) + sum_d w[c, taps - 1 - d] * x[t - d, c], d = 0 .. taps - 1, where rows
+// before the step's first come from the sequence's state (its last taps - 1 inputs, oldest first) and rows
+// before the sequence's start are zero (the state of a fresh slot is zero).  act 1: silu on the result.
+template <typename TO>
+__global__ void short_conv_kernel(const float* __restrict__ x, size_t x_stride, const float* __restrict__ w, int taps,
+                                  const float* __restrict__ state, const int32_t* __restrict__ tok_pos,
+                                  const int32_t* __restrict__ tok_seq, const int32_t* __restrict__ past_len,
+                                  const int32_t* __restrict__ slots, TO* __restrict__ out, size_t out_stride,
+                                  int residual, int act, int channels) {
+  const int t = blockIdx.x;
+  const int b = tok_seq[t];
+  const int pos = tok_pos[t], past = past_len[b];
+  const float* st = state + (size_t)slots[b] * (taps - 1) * channels;
+  for (int c = blockIdx.y * blockDim.x + threadIdx.x; c < channels; c += gridDim.y * blockDim.x) {
+    const float cur = x[(size_t)t * x_stride + c];
+    float acc = residual ? cur : 0.f;
+    for (int d = 0; d < taps; ++d) {
+      const int sp = pos - d;
+      float v;
+      if (sp >= past)
+        v = d == 0 ? cur : x[(size_t)(t - d) * x_stride + c];
+      else
+        v = st[(size_t)(sp - past + taps - 1) * channels + c];
+      acc = fmaf(w[(size_t)c * taps + (taps - 1 - d)], v, acc);
+    }
+    if (act == 1) acc = acc * rb_sigmoid(acc);
+    Num<TO>::store(out + (size_t)t * out_stride + c, acc);
+  }
+}
+
+extern "C" int rb_short_conv(const float* x, long long x_stride, const float* w, int taps, const float* state,
+                             const int32_t* tok_pos, const int32_t* tok_seq, const int32_t* past_len,
+                             const int32_t* slots, void* out, long long out_stride, int out_dtype, int residual,
+                             int act, int n_tokens, int channels, void* stream) {
+  RB_RECORDED(rb_short_conv(x, x_stride, w, taps, state, tok_pos, tok_seq, past_len, slots, out, out_stride, out_dtype,
+                            residual, act, n_tokens, channels, stream));
+  RB_REQUIRE(n_tokens >= 0 && channels > 0 && taps >= 1, "rb_short_conv: bad sizes T=%d C=%d taps=%d", n_tokens, channels, taps);
+  RB_REQUIRE(x_stride >= channels && out_stride >= channels, "rb_short_conv: a row stride is shorter than the channels");
+  RB_REQUIRE(taps == 1 || state != nullptr, "rb_short_conv: %d taps need a state", taps);
+  RB_REQUIRE(act == 0 || act == 1, "rb_short_conv: unknown activation %d", act);
+  if (n_tokens == 0) return 0;
+  dim3 grid(n_tokens, (channels + 255) / 256 < 16 ? (channels + 255) / 256 : 16);
+  hipStream_t s = (hipStream_t)stream;
+  if (out_dtype == RB_F32)
+    short_conv_kernel<float><<<grid, 256, 0, s>>>(x, (size_t)x_stride, w, taps, state, tok_pos, tok_seq, past_len, slots,
+                                                  (float*)out, (size_t)out_stride, residual, act, channels);
+  else if (out_dtype == RB_BF16)
+    short_conv_kernel<bf16_t><<<grid, 256, 0, s>>>(x, (size_t)x_stride, w, taps, state, tok_pos, tok_seq, past_len, slots,
+                                                   (bf16_t*)out, (size_t)out_stride, residual, act, channels);
+  else
+    RB_REQUIRE(false, "rb_short_conv: unknown dtype %d", out_dtype);
+  RB_LAUNCH_CHECK();
+  return 0;
+}
+
+// After the step: the state becomes the last taps - 1 inputs of the sequence, oldest first.  A thread owns a
+// channel of a sequence and reads all it needs before it writes.
+#define SC_MAX_TAPS 16
+__global__ void short_conv_state_kernel(const float* __restrict__ x, size_t x_stride, int taps, float* __restrict__ state,
+                                        const int32_t* __restrict__ cu_seqlens, const int32_t* __restrict__ slots,
+                                        int channels) {
+  const int b = blockIdx.x;
+  const int row0 = cu_seqlens[b], n = cu_seqlens[b + 1] - row0;
+  const int keep = taps - 1;
+  float* st = state + (size_t)slots[b] * keep * channels;
+  for (int c = blockIdx.y * blockDim.x + threadIdx.x; c < channels; c += gridDim.y * blockDim.x) {
+    float v[SC_MAX_TAPS];
+#pragma unroll
+    for (int i = 0; i < SC_MAX_TAPS; ++i) {
+      if (i < keep) {
+        const int r = n - keep + i;          // row of the step that lands in entry i; negative: an older input
+        v[i] = r >= 0 ? x[(size_t)(row0 + r) * x_stride + c] : st[(size_t)(i + n) * channels + c];
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < SC_MAX_TAPS; ++i)
+      if (i < keep) st[(size_t)i * channels + c] = v[i];
+  }
+}
+
+extern "C" int rb_short_conv_state(const float* x, long long x_stride, int taps, float* state, const int32_t* cu_seqlens,
+                                   const int32_t* slots, int n_seqs, int channels, void* stream) {
+  RB_RECORDED(rb_short_conv_state(x, x_stride, taps, state, cu_seqlens, slots, n_seqs, channels, stream));
+  RB_REQUIRE(n_seqs >= 0 && channels > 0 && taps >= 1 && taps - 1 <= SC_MAX_TAPS,
+             "rb_short_conv_state: bad sizes B=%d C=%d taps=%d (at most %d)", n_seqs, channels, taps, SC_MAX_TAPS + 1);
+  RB_REQUIRE(x_stride >= channels, "rb_short_conv_state: the row stride is shorter than the channels");
+  if (n_seqs == 0 || taps == 1) return 0;
+  dim3 grid(n_seqs, (channels + 255) / 256 < 64 ? (channels + 255) / 256 : 64);
+  short_conv_state_kernel<<<grid, 256, 0, (hipStream_t)stream>>>(x, (size_t)x_stride, taps, state, cu_seqlens, slots, channels);
+  RB_LAUNCH_CHECK();
+  return 0;
+}
+
+// ---------------------------------------------------------------- gated delta rule: what enters the recurrence
+// Per token, in place: every q and k head becomes a unit vector, x / sqrt(sum x^2 + unit_eps), q times q_scale;
+// a[t, h, i] becomes the decay exp(-exp(a_log[h]) * softplus(a + dt_bias[h, i])); beta[t, h] = sigmoid(b[t, h]).
+__global__ void delta_prep_kernel(float* __restrict__ qk, size_t qk_stride, int n_kv, int dim, float* __restrict__ a,
+                                  size_t a_stride, const float* __restrict__ dt_bias, const float* __restrict__ a_log, int n_heads,
+                                  const float* __restrict__ b_in, size_t b_stride, float* __restrict__ beta,
+                                  float q_scale, float unit_eps) {
+  const int t = blockIdx.x;
+  const int lane = threadIdx.x & (RB_WAVE - 1);
+  const int wave = threadIdx.x / RB_WAVE, n_waves = blockDim.x / RB_WAVE;
+  float* row = qk + (size_t)t * qk_stride;
+  for (int v = wave; v < 2 * n_kv; v += n_waves) {           // the q heads, then the k heads
+    float* p = row + (size_t)v * dim;
+    float ss = 0.f;
+    for (int i = lane; i < dim; i += RB_WAVE) ss = fmaf(p[i], p[i], ss);
+    ss = wave_sum(ss);
+    const float f = (v < n_kv ? q_scale : 1.0f) / sqrtf(ss + unit_eps);
+    for (int i = lane; i < dim; i += RB_WAVE) p[i] *= f;
+  }
+  float* ar = a + (size_t)t * a_stride;
+  for (int i = threadIdx.x; i < n_heads * dim; i += blockDim.x) {
+    const int h = i / dim;
+    ar[i] = expf(-expf(a_log[h]) * rb_softplus(ar[i] + dt_bias[i]));
+  }
+  for (int h = threadIdx.x; h < n_heads; h += blockDim.x) beta[(size_t)t * n_heads + h] = rb_sigmoid(b_in[(size_t)t * b_stride + h]);
+}
+
+extern "C" int rb_delta_prep(float* qk, long long qk_stride, int n_kv_heads, int dim, float* a, long long a_stride, const float* dt_bias,
+                             const float* a_log, int n_heads, const float* b_in, long long b_stride, float* beta,
+                             float q_scale, float unit_eps, int n_tokens, void* stream) {
+  RB_RECORDED(rb_delta_prep(qk, qk_stride, n_kv_heads, dim, a, a_stride, dt_bias, a_log, n_heads, b_in, b_stride, beta, q_scale,
+                            unit_eps, n_tokens, stream));
+  RB_REQUIRE(n_tokens >= 0 && n_kv_heads > 0 && n_heads > 0 && dim > 0, "rb_delta_prep: bad sizes");
+  RB_REQUIRE(qk_stride >= 2LL * n_kv_heads * dim && b_stride >= n_heads && a_stride >= (long long)n_heads * dim,
+             "rb_delta_prep: a row stride is too short");
+  if (n_tokens == 0) return 0;
+  delta_prep_kernel<<<n_tokens, 256, 0, (hipStream_t)stream>>>(qk, (size_t)qk_stride, n_kv_heads, dim, a, (size_t)a_stride, dt_bias, a_log,
+                                                               n_heads, b_in, (size_t)b_stride, beta, q_scale, unit_eps);
+  RB_LAUNCH_CHECK();
+  return 0;
+}
+
+// ---------------------------------------------------------------- gated delta rule: the recurrence
+// Per sequence and head, token after token:
+//   S <- diag(g) S;  u = beta (v - S^T k);  S <- S + k u^T;  o = S^T q
+// The columns of S (one per value channel) do not meet: a column is held by RG lanes, each with DKL of its rows in
+// registers; the two dot products over the rows are finished by shuffles among the RG lanes.  A wave holds 64 / RG
+// columns; q, k and g of a few tokens are staged in LDS for all lanes.  The state is read once and written once.
+#define DR_CHUNK 8
+template <int DKL, int RG>
+__global__ __launch_bounds__(RB_WAVE) void delta_rule_kernel(
+    const float* __restrict__ q, const float* __restrict__ k, size_t qk_stride, const float* __restrict__ v,
+    size_t v_stride, const float* __restrict__ g, size_t g_stride, const float* __restrict__ beta, float* __restrict__ state,
+    const int32_t* __restrict__ cu_seqlens, const int32_t* __restrict__ slots, float* __restrict__ out, int n_heads,
+    int n_kv, int dim, int vdim) {
+  constexpr int COLS = RB_WAVE / RG;
+  constexpr int DK = DKL * RG;               // rows held, >= dim; rows beyond dim stay zero
+  __shared__ float sq[DR_CHUNK][DK], sk[DR_CHUNK][DK], sg[DR_CHUNK][DK];
+  const int b = blockIdx.x, h = blockIdx.y;
+  const int lane = threadIdx.x;
+  const int col = blockIdx.z * COLS + lane / RG;
+  const int rg = lane % RG;
+  const bool on = col < vdim;
+  const int kvh = h / (n_heads / n_kv);
+  const int row0 = cu_seqlens[b], n = cu_seqlens[b + 1] - row0;
+  float* S = state + (((size_t)slots[b] * n_heads + h) * dim) * vdim;
+  float s[DKL];
+#pragma unroll
+  for (int i = 0; i < DKL; ++i) {
+    const int r = rg * DKL + i;
+    s[i] = (on && r < dim) ? S[(size_t)r * vdim + col] : 0.f;
+  }
+  for (int t0 = 0; t0 < n; t0 += DR_CHUNK) {
+    const int nt = n - t0 < DR_CHUNK ? n - t0 : DR_CHUNK;
+    __builtin_amdgcn_s_barrier();
+    for (int idx = lane; idx < nt * DK; idx += RB_WAVE) {
+      const int tt = idx / DK, i = idx - tt * DK;
+      const size_t t = (size_t)(row0 + t0 + tt);
+      const bool in = i < dim;
+      sq[tt][i] = in ? q[t * qk_stride + (size_t)kvh * dim + i] : 0.f;
+      sk[tt][i] = in ? k[t * qk_stride + (size_t)kvh * dim + i] : 0.f;
+      sg[tt][i] = in ? g[t * g_stride + (size_t)h * dim + i] : 0.f;
+    }
+    __builtin_amdgcn_s_barrier();
+    for (int tt = 0; tt < nt; ++tt) {
+      const size_t t = (size_t)(row0 + t0 + tt);
+      const float vv = on ? v[t * v_stride + (size_t)h * vdim + col] : 0.f;
+      const float bt = beta[t * n_heads + h];
+      float kv = 0.f;
+#pragma unroll
+      for (int i = 0; i < DKL; ++i) {
+        s[i] *= sg[tt][rg * DKL + i];
+        kv = fmaf(s[i], sk[tt][rg * DKL + i], kv);
+      }
+#pragma unroll
+      for (int o = 1; o < RG; o <<= 1) kv += __shfl_xor(kv, o, RB_WAVE);
+      const float u = bt * (vv - kv);
+      float oq = 0.f;
+#pragma unroll
+      for (int i = 0; i < DKL; ++i) {
+        s[i] = fmaf(sk[tt][rg * DKL + i], u, s[i]);
+        oq = fmaf(s[i], sq[tt][rg * DKL + i], oq);
+      }
+#pragma unroll
+      for (int o = 1; o < RG; o <<= 1) oq += __shfl_xor(oq, o, RB_WAVE);
+      if (on && rg == 0) out[(t * n_heads + h) * vdim + col] = oq;
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < DKL; ++i) {
+    const int r = rg * DKL + i;
+    if (on && r < dim) S[(size_t)r * vdim + col] = s[i];
+  }
+}
+
+template <int DKL, int RG>
+static void launch_delta_rule(const float* q, const float* k, size_t qk_stride, const float* v, size_t v_stride,
+                              const float* g, size_t g_stride, const float* beta, float* state, const int32_t* cu_seqlens,
+                              const int32_t* slots, float* out, int n_seqs, int n_heads, int n_kv, int dim, int vdim,
+                              hipStream_t s) {
+  constexpr int COLS = RB_WAVE / RG;
+  dim3 grid(n_seqs, n_heads, (vdim + COLS - 1) / COLS);
+  delta_rule_kernel<DKL, RG><<<grid, RB_WAVE, 0, s>>>(q, k, qk_stride, v, v_stride, g, g_stride, beta, state, cu_seqlens, slots,
+                                                      out, n_heads, n_kv, dim, vdim);
+}
+
+extern "C" int rb_delta_rule(const float* q, const float* k, long long qk_stride, const float* v, long long v_stride,
+                             const float* g, long long g_stride, const float* beta, float* state, const int32_t* cu_seqlens,
+                             const int32_t* slots, float* out, int n_seqs, int n_heads, int n_kv_heads, int dim, int vdim,
+                             void* stream) {
+  RB_RECORDED(rb_delta_rule(q, k, qk_stride, v, v_stride, g, g_stride, beta, state, cu_seqlens, slots, out, n_seqs, n_heads,
+                            n_kv_heads, dim, vdim, stream));
+  RB_REQUIRE(n_seqs >= 0 && n_heads > 0 && n_kv_heads > 0 && n_heads % n_kv_heads == 0 && dim > 0 && vdim > 0,
+             "rb_delta_rule: bad sizes H=%d Hk=%d dim=%d vdim=%d", n_heads, n_kv_heads, dim, vdim);
+  RB_REQUIRE(g_stride >= (long long)n_heads * dim, "rb_delta_rule: the decays' row stride is too short");
+  RB_REQUIRE(dim <= 512, "rb_delta_rule: key size %d not supported (at most 512)", dim);
+  RB_REQUIRE(n_heads <= 65535 && vdim <= 65535 * 4, "rb_delta_rule: too many heads or value channels");
+  if (n_seqs == 0) return 0;
+  hipStream_t s = (hipStream_t)stream;
+  const size_t qs = (size_t)qk_stride, vs = (size_t)v_stride;
+#define DR_GO(DKL, RG) \
+  launch_delta_rule<DKL, RG>(q, k, qs, v, vs, g, (size_t)g_stride, beta, state, cu_seqlens, slots, out, n_seqs, n_heads, n_kv_heads, dim, vdim, s)
+  // rows of a column over RG lanes: short chains per token, and enough waves for the GPU while sequences are few
+  if (dim <= 16)
+    DR_GO(4, 4);
+  else if (dim <= 32)
+    DR_GO(8, 4);
+  else if (dim <= 64)
+    DR_GO(8, 8);
+  else if (dim <= 128)
+    DR_GO(16, 8);
+  else if (dim <= 256)
+    DR_GO(16, 16);
+  else
+    DR_GO(32, 16);
+#undef DR_GO
+  RB_LAUNCH_CHECK();
+  return 0;
+}
+
+// ---------------------------------------------------------------- read-out norm with gate
+// out[t, h, :] = o[t, h, :] / sqrt(mean(o^2) + eps) * weight * sigmoid(gate[t, h, :]); a wave per (token, head).
+template <typename TO>
+__global__ void gated_rmsnorm_kernel(const float* __restrict__ o, const float* __restrict__ weight,
+                                     const float* __restrict__ gate, size_t gate_stride, float eps, TO* __restrict__ out,
+                                     int n_heads, int vdim, long long n_pairs) {
+  const long long pair = (long long)blockIdx.x * (blockDim.x / RB_WAVE) + threadIdx.x / RB_WAVE;
+  if (pair >= n_pairs) return;
+  const int lane = threadIdx.x & (RB_WAVE - 1);
+  const size_t t = (size_t)(pair / n_heads);
+  const int h = (int)(pair % n_heads);
+  const float* p = o + (size_t)pair * vdim;
+  const float* gp = gate + t * gate_stride + (size_t)h * vdim;
+  float ss = 0.f;
+  for (int i = lane; i < vdim; i += RB_WAVE) ss = fmaf(p[i], p[i], ss);
+  ss = wave_sum(ss);
+  const float f = 1.0f / sqrtf(ss / (float)vdim + eps);
+  for (int i = lane; i < vdim; i += RB_WAVE)
+    Num<TO>::store(out + (size_t)pair * vdim + i, p[i] * f * weight[i] * rb_sigmoid(gp[i]));
+}
+
+extern "C" int rb_gated_rmsnorm(const float* o, const float* weight, const float* gate, long long gate_stride, float eps,
+                                void* out, int out_dtype, int n_tokens, int n_heads, int vdim, void* stream) {
+  RB_RECORDED(rb_gated_rmsnorm(o, weight, gate, gate_stride, eps, out, out_dtype, n_tokens, n_heads, vdim, stream));
+  RB_REQUIRE(n_tokens >= 0 && n_heads > 0 && vdim > 0, "rb_gated_rmsnorm: bad sizes");
+  RB_REQUIRE(gate_stride >= (long long)n_heads * vdim, "rb_gated_rmsnorm: the gate's row stride is too short");
+  if (n_tokens == 0) return 0;
+  const long long n_pairs = (long long)n_tokens * n_heads;
+  const int grid = (int)((n_pairs + 3) / 4);
+  hipStream_t s = (hipStream_t)stream;
+  if (out_dtype == RB_F32)
+    gated_rmsnorm_kernel<float><<<grid, 256, 0, s>>>(o, weight, gate, (size_t)gate_stride, eps, (float*)out, n_heads, vdim, n_pairs);
+  else if (out_dtype == RB_BF16)
+    gated_rmsnorm_kernel<bf16_t><<<grid, 256, 0, s>>>(o, weight, gate, (size_t)gate_stride, eps, (bf16_t*)out, n_heads, vdim, n_pairs);
+  else
+    RB_REQUIRE(false, "rb_gated_rmsnorm: unknown dtype %d", out_dtype);
+  RB_LAUNCH_CHECK();
+  return 0;
+}

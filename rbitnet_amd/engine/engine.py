@@ -134,7 +134,9 @@ class Engine:
         """A model folder (config.json + model.safetensors), as the reference's
         `Engine::load_path` takes a GGUF path (inference.rs:121-133)."""
         from ..weights.safetensors_io import WeightFolder
-        cfg, spec = load_config(path, tensor_names=WeightFolder(path).names())
+        store = WeightFolder(path)
+        cfg, spec = load_config(path, tensor_names=store.names(),
+                                tensor_shapes={name: tuple(store.info(name)[1]) for name in store.names()})
 
         def tensors_for(model: Model, cfg):
             aliases = getattr(type(cfg), "tensor_aliases", None)

@@ -34,12 +34,19 @@ def _ends(spec: ModelSpec, env: BuildEnv):
     return build_part("embedding", spec.embedding, env), build_part("head", spec.head, env)
 
 
+def _join(*pieces: str) -> str:
+    """A tensor's name from its layer's prefix, its part's segment and the part's own name for it; any of them
+    may be empty (a layer's own tensors have no segment, a norm's weight may be named like the norm)."""
+    return ".".join(p for p in pieces if p)
+
+
 def _named_parts(spec: ModelSpec, blocks) -> Dict[str, object]:
     """prefix -> part, for every part of a block that owns tensors (the two ends name theirs in full)."""
     out: Dict[str, object] = {}
     for layer, block in zip(spec.layers, blocks):
         for segment, part in block.parts().items():
-            out[f"{layer.prefix}.{segment}"] = part
+            if part is not None:
+                out[_join(layer.prefix, segment)] = part
     return out
 
 
@@ -49,7 +56,7 @@ def _expected(spec: ModelSpec, blocks, embedding, head) -> Dict[str, TensorSpec]
         out.update(part.tensor_specs())
     for prefix, part in _named_parts(spec, blocks).items():
         for name, ts in part.tensor_specs().items():
-            out[f"{prefix}.{name}"] = ts
+            out[_join(prefix, name)] = ts
     return out
 
 
@@ -86,12 +93,16 @@ class Model:
         self.expected = _expected(spec, self.blocks, self.embedding, self.head)
 
     # ------------------------------------------------------------------ cache needs
-    def cache_requests(self) -> List[Optional[CacheRequest]]:
+    def cache_requests(self) -> List:
         """One entry per place in the schedule: a layer that runs twice keeps two caches,
         since its second run sees other inputs than its first."""
         out = []
         for i in self.spec.schedule:
-            req = getattr(self.blocks[i].mixer, "cache_request", None)
+            block = self.blocks[i]
+            if hasattr(block, "cache_requests"):          # a block with needs of its own says all of them
+                out.append(block.cache_requests())
+                continue
+            req = getattr(block.mixer, "cache_request", None)
             out.append(req() if req else None)
         return out
 
@@ -153,7 +164,7 @@ class Model:
         self.embedding.load({name: placed(name) for name in self.embedding.tensor_specs()})
         self.head.load({name: placed(name) for name in self.head.tensor_specs()}, embedding=self.embedding)
         for prefix, part in _named_parts(self.spec, self.blocks).items():
-            part.load({name: placed(f"{prefix}.{name}") for name in part.tensor_specs()})
+            part.load({name: placed(_join(prefix, name)) for name in part.tensor_specs()})
 
     def weight_bytes(self) -> int:
         """Bytes of every weight a step reads once: all tensors of the blocks, and of the two ends

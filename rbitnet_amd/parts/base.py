@@ -64,7 +64,10 @@ class CacheRequest:
                   behind it can be given back.
     kind "state": `state_shape` numbers per sequence, set to `state_init` when a
                   slot is handed out.
-    Layers with equal requests share one group of storage."""
+    Layers with equal requests share one group of storage.  A layer may ask for several things
+    (a list of requests); `name` tells them apart: a state is found at `view.states[name]`.
+    `values = False` (kind "kv"): the layer stores one vector per token that serves as key and
+    value at once, so no second set of pages is kept and `view.v_pages` is `view.k_pages`."""
     kind: str
     heads: int = 0
     head_dim: int = 0
@@ -72,10 +75,12 @@ class CacheRequest:
     state_shape: Tuple[int, ...] = ()
     state_init: float = 0.0
     state_dtype: torch.dtype = torch.float32
+    name: str = ""
+    values: bool = True
 
     def key(self) -> Tuple:
         return (self.kind, self.heads, self.head_dim, self.window, tuple(self.state_shape),
-                self.state_init, self.state_dtype)
+                self.state_init, self.state_dtype, self.name, self.values)
 
 
 class Part:

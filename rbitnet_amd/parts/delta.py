@@ -1,0 +1,125 @@
+"""The gated delta rule with a decay per key channel: a recurrent mixer whose state is, per head, a matrix
+S [key dim, value dim] in float32.
+
+Per token, with h the mixer's input:
+    q, k = Wq h, Wk h  (kv_heads x dim each);  v = Wv h  (heads x vdim);  head i reads q/k head i // (heads // kv_heads)
+    each of q, k, v: short causal convolution per channel, then silu
+    q, k: unit vectors per head, x / sqrt(sum x^2 + 1e-6);  q also times dim^(-1/2)
+    beta = sigmoid(Wb h)                                          one per head
+    g = exp(-exp(A_log[head]) * softplus(Wa2 (Wa1 h) + dt_bias))  one per head and key channel
+    S <- diag(g) S;  u = beta (v - S^T k);  S <- S + k u^T;  o = S^T q          (the read-out sees the token's own write)
+    o <- o / sqrt(mean(o^2) + eps) * norm * sigmoid(Wg2 (Wg1 h));   out = Wo o
+
+In float32: everything from the unit vectors on (decays, beta, the recurrence, the read-out norm and its gate); the
+projections and the convolution's inputs are float32 sums of products in the compute dtype.  The state and the
+convolution's last taps - 1 inputs live in the cache (`view.states["delta"]`, `view.states["conv"]`).
+
+Parameters: heads, kv_heads, dim, vdim, conv (taps), eps (of the read-out norm), unit_eps (1e-6), low-rank sizes come
+from the tensors' declared shapes: decay_rank, gate_rank.  names: the tensors below the layer's prefix.
+"""
+from __future__ import annotations
+
+from typing import Dict, List, Optional
+
+import torch
+
+from ..errors import ConfigError
+from .base import BuildEnv, CacheRequest, Part, TensorSpec, register_mixer
+from .linear import linear, pack_rows
+from .short_conv import ACT_SILU, ShortConv
+
+DEFAULT_NAMES = {"q": "q", "k": "k", "v": "v", "q_conv": "q.conv", "k_conv": "k.conv", "v_conv": "v.conv", "b": "b",
+                 "a_log": "A_log", "norm": "norm", "a1": "a1", "a2": "a2", "dt_bias": "dt_bias", "g1": "g1", "g2": "g2",
+                 "o": "o"}
+
+
+class ChannelDelta(Part):
+    graph_safe = True
+    plan_safe = True
+
+    def __init__(self, params: Dict, env: BuildEnv):
+        self.env = env
+        self.heads = int(params["heads"])
+        self.kv_heads = int(params.get("kv_heads") or self.heads)
+        self.dim, self.vdim = int(params["dim"]), int(params["vdim"])
+        self.taps = int(params["conv"])
+        self.eps = float(params["eps"])
+        self.unit_eps = float(params.get("unit_eps", 1e-6))
+        self.decay_rank, self.gate_rank = int(params["decay_rank"]), int(params["gate_rank"])
+        if self.heads <= 0 or self.kv_heads <= 0 or self.heads % self.kv_heads != 0:
+            raise ConfigError(f"delta rule: {self.heads} heads cannot share {self.kv_heads} q/k heads")
+        if not 0 < self.dim <= 512:
+            raise ConfigError(f"delta rule: key size {self.dim} not supported (1 to 512)")
+        self.names = dict(DEFAULT_NAMES, **(params.get("names") or {}))
+        self.hidden = env.hidden_size
+        self.n_qk, self.n_v = self.kv_heads * self.dim, self.heads * self.vdim
+        self.n_conv = 2 * self.n_qk + self.n_v
+        self.conv = ShortConv(self.n_conv, self.taps, env, residual=False, act=ACT_SILU)
+        self.cache_from = None
+
+    # ------------------------------------------------------------------ tensors
+    def tensor_specs(self) -> Dict[str, TensorSpec]:
+        n, e = self.names, self.hidden
+        gain = lambda *shape: TensorSpec(tuple(shape), role="gain", init="normal")
+        return {
+            n["q"]: TensorSpec((self.n_qk, e)), n["k"]: TensorSpec((self.n_qk, e)), n["v"]: TensorSpec((self.n_v, e)),
+            n["q_conv"]: gain(self.n_qk, self.taps), n["k_conv"]: gain(self.n_qk, self.taps),
+            n["v_conv"]: gain(self.n_v, self.taps),
+            n["b"]: TensorSpec((self.heads, e)), n["a_log"]: gain(self.heads),
+            n["norm"]: TensorSpec((self.vdim,), role="gain", init="ones_normal"),
+            n["a1"]: TensorSpec((self.decay_rank, e)), n["a2"]: TensorSpec((self.heads * self.dim, self.decay_rank)),
+            n["dt_bias"]: gain(self.heads * self.dim),
+            n["g1"]: TensorSpec((self.gate_rank, e)), n["g2"]: TensorSpec((self.n_v, self.gate_rank)),
+            n["o"]: TensorSpec((e, self.n_v)),
+        }
+
+    def load(self, tensors: Dict[str, torch.Tensor]) -> None:
+        lib, allowed, n = self.env.lib, not getattr(self.env, "generic_only", False), self.names
+        first = tensors[n["q"]]
+        # one product for q, k, v and beta, one for the two low-rank inputs
+        pieces, row = [], 0
+        for key in ("q", "k", "v", "b"):
+            pieces.append((tensors[n[key]], row, None, None))
+            row += tensors[n[key]].shape[0]
+        self.w_in = pack_rows(lib, pieces, row, self.hidden, first.dtype, first.device, allowed)
+        self.b_col = self.n_conv
+        low = [(tensors[n["a1"]], 0, None, None), (tensors[n["g1"]], self.decay_rank, None, None)]
+        self.w_low = pack_rows(lib, low, self.decay_rank + self.gate_rank, self.hidden, first.dtype, first.device, allowed)
+        # the second halves as one block-diagonal matrix: [a | gate] = [a1 h | g1 h] W^T
+        r = self.decay_rank + self.gate_rank
+        up = torch.zeros((self.heads * self.dim + self.n_v, r), dtype=first.dtype, device=first.device)
+        up[:self.heads * self.dim, :self.decay_rank] = tensors[n["a2"]]
+        up[self.heads * self.dim:, self.decay_rank:] = tensors[n["g2"]]
+        self.w_up = pack_rows(lib, [(up, 0, None, None)], up.shape[0], r, first.dtype, first.device, allowed)
+        self.conv.load(torch.cat([tensors[n["q_conv"]], tensors[n["k_conv"]], tensors[n["v_conv"]]]))
+        self.a_log, self.dt_bias, self.norm = tensors[n["a_log"]], tensors[n["dt_bias"]], tensors[n["norm"]]
+        o = tensors[n["o"]]
+        self.w_o = pack_rows(lib, [(o, 0, None, None)], o.shape[0], o.shape[1], o.dtype, o.device, allowed)
+
+    def cache_requests(self) -> List[CacheRequest]:
+        out = [CacheRequest("state", state_shape=(self.heads, self.dim, self.vdim), state_init=0.0, name="delta")]
+        conv = self.conv.cache_request("conv")
+        return out + ([conv] if conv else [])
+
+    def cache_request(self) -> Optional[CacheRequest]:
+        return self.cache_requests()[0]
+
+    # ------------------------------------------------------------------ forward
+    def forward(self, h: torch.Tensor, ctx, view, stream: Optional[torch.Tensor] = None, next_norm=None) -> torch.Tensor:
+        lib, t = self.env.lib, h.shape[0]
+        proj = linear(lib, h, self.w_in, torch.float32)                       # [T, q | k | v | b]
+        low = linear(lib, h, self.w_low, self.env.dtype)                      # [T, a1 h | g1 h]
+        up = linear(lib, low, self.w_up, torch.float32)                       # [T, a | gate]
+        qkv = self.conv.forward(proj, ctx, view.states.get("conv"), torch.float32)
+        n_a = self.heads * self.dim
+        beta = torch.empty((t, self.heads), dtype=torch.float32, device=h.device)
+        lib.delta_prep(qkv, self.kv_heads, self.dim, up, self.dt_bias, self.a_log, self.heads, proj, self.b_col, beta,
+                       self.dim ** -0.5, self.unit_eps)
+        o = torch.empty((t, self.n_v), dtype=torch.float32, device=h.device)
+        lib.delta_rule(qkv, self.kv_heads, self.dim, self.heads, self.vdim, up, beta, view.states["delta"], ctx, o)
+        on = torch.empty((t, self.n_v), dtype=self.env.dtype, device=h.device)
+        lib.gated_rmsnorm(o, self.norm, up, n_a, self.eps, self.heads, self.vdim, on)
+        return linear(lib, on, self.w_o, torch.float32)
+
+
+register_mixer("channel_delta", ChannelDelta)

@@ -7,13 +7,15 @@ caps its logits, or computes them in another way, registers another kind.
 Their tensors have no layer prefix: `tensor_specs` names them in full.
 
 embedding "table" (crates/bitnet-core/src/llama/model.rs:229-232): x[t, :] = table[id[t], :].
-    Parameters: name, vocab_size.
+    Parameters: name, vocab_size, streams (None: the stream is [T, E]; n: n equal copies [n, T, E], for
+    blocks that keep the residual stream in several copies).
     Interface of an embedding: tensor_specs() / load(tensors) / forward(ctx) -> float32 [T, E]
     (ctx.token_ids int32 [T]); `table` if a head may share it.
 
 head "linear" (model.rs:309-315): logits = W norm(x), on the asked rows only; W is the
     embedding's table when the parameters name no matrix (tied).
-    Parameters: norm (a PartSpec), norm_name, name (None: tied), vocab_size.
+    Parameters: norm (a PartSpec), norm_name, name (None: tied), vocab_size, softcap (None, or c:
+    logits <- c tanh(logits / c)).  A stream in several copies is summed by the norm.
     Interface of a head: tensor_specs() / load(tensors, embedding) /
     forward(x, pending, rows, ctx) -> float32 [len(rows), V], where x is the stream, `pending`
     what the last block left to be added (see stream.py) and rows the packed rows asked for;
@@ -42,6 +44,7 @@ class TableEmbedding(Part):
         self.name = str(params["name"])
         self.vocab_size = int(params["vocab_size"])
         self.hidden = env.hidden_size
+        self.streams = None if params.get("streams") is None else int(params["streams"])
         self.table: Optional[torch.Tensor] = None
 
     def tensor_specs(self) -> Dict[str, TensorSpec]:
@@ -54,6 +57,10 @@ class TableEmbedding(Part):
         return 0                      # the gather reads a few rows only
 
     def forward(self, ctx) -> torch.Tensor:
+        if self.streams is not None:
+            x = torch.empty((self.streams, ctx.n_tokens, self.hidden), dtype=torch.float32, device=self.table.device)
+            self.env.lib.embed_streams(self.table, ctx.token_ids, x)
+            return x
         x = torch.empty((ctx.n_tokens, self.hidden), dtype=torch.float32, device=self.table.device)
         self.env.lib.embed_gather(self.table, ctx.token_ids, x)
         return x
@@ -69,6 +76,9 @@ class LinearHead(Part):
         self.name = params.get("name")
         self.vocab_size = int(params["vocab_size"])
         self.hidden = env.hidden_size
+        self.softcap = None if params.get("softcap") is None else float(params["softcap"])
+        if self.softcap is not None and not self.softcap > 0:
+            raise ConfigError(f"a head's softcap must be positive, found {self.softcap}")
         self.weight = None
 
     @property
@@ -86,6 +96,8 @@ class LinearHead(Part):
     def _norm_names(self) -> Dict[str, str]:
         """full name -> the norm's own name of the tensor"""
         specs = self.norm.tensor_specs()
+        if hasattr(self.norm, "tensor_names"):
+            return self.norm.tensor_names(self.norm_name)
         if len(specs) == 1:
             return {self.norm_name: next(iter(specs))}
         base = self.norm_name.rsplit(".", 1)[0]
@@ -116,7 +128,10 @@ class LinearHead(Part):
 
     def forward(self, x: torch.Tensor, pending, rows: torch.Tensor, ctx=None) -> torch.Tensor:
         xn = normed_for(self, self.norm, x, pending, rows)
-        return linear(self.env.lib, xn, self.weight, torch.float32)
+        logits = linear(self.env.lib, xn, self.weight, torch.float32)
+        if self.softcap is not None:
+            self.env.lib.tanh_cap(logits, self.softcap)
+        return logits
 
 
 def _numel(shape) -> int:

@@ -18,7 +18,7 @@ import torch
 
 from ..errors import ConfigError
 from .base import BuildEnv, Part, TensorSpec, register_feed_forward
-from .linear import can_fuse_gate, gated_linear, linear_to_stream, pack_gate_up, pack_rows
+from .linear import can_fuse_gate, gated_linear, linear, linear_to_stream, pack_gate_up, pack_rows
 
 DEFAULT_NAMES = {"gate": "gate_proj.weight", "up": "up_proj.weight", "down": "down_proj.weight"}
 
@@ -59,4 +59,38 @@ class SwiGLU(Part):
         return linear_to_stream(lib, t, self.w_down, stream, next_norm)
 
 
+class DenseXielu(Part):
+    """out = Wdown act(Wup h) with act = xIELU: for z > 0, softplus(p) z^2 + z / 2; for z <= 0,
+    (1/2 + softplus(q)) (exp(z) - 1 - z) + z / 2, (p, q) being the two numbers of the tensor `act`.
+    Parameters: intermediate_size, names ({"up", "down", "act"})."""
+    graph_safe = True
+    plan_safe = True
+
+    def __init__(self, params: Dict, env: BuildEnv):
+        self.env = env
+        self.ff = int(params["intermediate_size"])
+        self.names = dict({"up": "up", "down": "down", "act": "act"}, **(params.get("names") or {}))
+        self.hidden = env.hidden_size
+
+    def tensor_specs(self) -> Dict[str, TensorSpec]:
+        return {self.names["up"]: TensorSpec((self.ff, self.hidden)), self.names["down"]: TensorSpec((self.hidden, self.ff)),
+                self.names["act"]: TensorSpec((2,), role="gain", init="normal")}
+
+    def load(self, tensors: Dict[str, torch.Tensor]) -> None:
+        allowed = not getattr(self.env, "generic_only", False)
+        up, down = tensors[self.names["up"]], tensors[self.names["down"]]
+        self.w_up = pack_rows(self.env.lib, [(up, 0, None, None)], up.shape[0], up.shape[1], up.dtype, up.device, allowed)
+        self.w_down = pack_rows(self.env.lib, [(down, 0, None, None)], down.shape[0], down.shape[1], down.dtype,
+                                down.device, allowed)
+        self.act = tensors[self.names["act"]]
+
+    def forward(self, h, ctx=None, stream: Optional[torch.Tensor] = None, next_norm=None):
+        lib = self.env.lib
+        z = linear(lib, h, self.w_up, torch.float32)
+        t = torch.empty((h.shape[0], self.ff), dtype=self.env.dtype, device=z.device)
+        lib.xielu(z, self.act, t)
+        return linear(lib, t, self.w_down, torch.float32)
+
+
 register_feed_forward("swiglu", SwiGLU)
+register_feed_forward("dense_xielu", DenseXielu)

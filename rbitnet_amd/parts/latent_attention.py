@@ -1,0 +1,107 @@
+"""Causal attention through a latent, without positions, with a sink in the softmax.
+
+Per token, with h the mixer's input (all norms RMS norms with a plain weight):
+    cq = norm(Wdq h),  q = Wuq cq              (heads x dim)
+    c  = norm(Wdkv h)                           (kv_rank numbers: all that is cached of a token)
+    per head i:  k_j = Wuk_i c_j,  v_j = Wuv_i c_j,  score_ij = (q_i . k_j) * scale  over the tokens j <= the query's
+    weights = exp(score) / (sum_j exp(score_j) + exp(sink_i)): the sink has no key and no value and is not scaled
+    out = Wo [sum_j weights_j v_j]_heads
+A layer with `cache_from = j` has no Wdkv: it reads the latents that layer j stored, with matrices of its own.
+
+The products with Wuk and Wuv are moved to the query's side, so that attention runs over the cached latents
+themselves, one key/value head of size kv_rank shared by all query heads:
+    score = (Wuk_i^T q_i) . c_j,      sum_j w_j v_j = Wuv_i (sum_j w_j c_j)
+which costs a product per head on either side of attention (`heads_linear`) and never expands the cache, whatever
+the step brings on top of whatever past.  Scores, softmax and norms in float32.
+
+Parameters: heads, dim, vdim, q_rank, kv_rank, scale, eps, cache_from, names.
+"""
+from __future__ import annotations
+
+from typing import Dict, Optional
+
+import torch
+
+from ..errors import ConfigError
+from .base import BuildEnv, CacheRequest, Part, TensorSpec, register_mixer
+from .linear import linear, pack_rows
+
+DEFAULT_NAMES = {"dq": "dq", "dq_norm": "dq.norm", "uq": "uq", "dkv": "dkv", "dkv_norm": "dkv.norm", "uk": "uk", "uv": "uv",
+                 "sink": "sink", "o": "o"}
+MAX_RANK = 256             # the attention kernel's largest head size
+
+
+class LatentAttention(Part):
+    graph_safe = True
+    plan_safe = True
+
+    def __init__(self, params: Dict, env: BuildEnv):
+        self.env = env
+        self.heads, self.dim, self.vdim = int(params["heads"]), int(params["dim"]), int(params["vdim"])
+        self.q_rank, self.kv_rank = int(params["q_rank"]), int(params["kv_rank"])
+        self.scale = float(params["scale"])
+        self.eps = float(params["eps"])
+        self.cache_from = params.get("cache_from")
+        self.window = None
+        if self.kv_rank <= 0 or self.kv_rank % 2 != 0 or self.kv_rank > MAX_RANK:
+            raise ConfigError(f"latent attention: kv_rank {self.kv_rank} not supported (even, at most {MAX_RANK})")
+        if min(self.heads, self.dim, self.vdim, self.q_rank) <= 0:
+            raise ConfigError("latent attention: sizes must be positive")
+        self.names = dict(DEFAULT_NAMES, **(params.get("names") or {}))
+        self.hidden = env.hidden_size
+
+    def tensor_specs(self) -> Dict[str, TensorSpec]:
+        n, e = self.names, self.hidden
+        gain = lambda size: TensorSpec((size,), role="gain", init="ones_normal")
+        out = {n["dq"]: TensorSpec((self.q_rank, e)), n["dq_norm"]: gain(self.q_rank),
+               n["uq"]: TensorSpec((self.heads * self.dim, self.q_rank)),
+               n["uk"]: TensorSpec((self.heads * self.dim, self.kv_rank)),
+               n["uv"]: TensorSpec((self.heads * self.vdim, self.kv_rank)),
+               n["sink"]: TensorSpec((self.heads,), role="gain", init="normal"),
+               n["o"]: TensorSpec((e, self.heads * self.vdim))}
+        if self.cache_from is None:
+            out[n["dkv"]] = TensorSpec((self.kv_rank, e))
+            out[n["dkv_norm"]] = gain(self.kv_rank)
+        return out
+
+    def load(self, tensors: Dict[str, torch.Tensor]) -> None:
+        lib, allowed, n = self.env.lib, not getattr(self.env, "generic_only", False), self.names
+        owns = self.cache_from is None
+        pieces = [(tensors[n["dq"]], 0, None, None)] + ([(tensors[n["dkv"]], self.q_rank, None, None)] if owns else [])
+        first = tensors[n["dq"]]
+        rows = self.q_rank + (self.kv_rank if owns else 0)
+        self.w_down = pack_rows(lib, pieces, rows, self.hidden, first.dtype, first.device, allowed)
+        self.q_gain = tensors[n["dq_norm"]]
+        self.kv_gain = tensors[n["dkv_norm"]] if owns else None
+        uq, o = tensors[n["uq"]], tensors[n["o"]]
+        self.w_uq = pack_rows(lib, [(uq, 0, None, None)], uq.shape[0], uq.shape[1], uq.dtype, uq.device, allowed)
+        self.w_o = pack_rows(lib, [(o, 0, None, None)], o.shape[0], o.shape[1], o.dtype, o.device, allowed)
+        # per head, stored [inner, outer]: Wuk_i [dim, rank] as it is (q_i -> Wuk_i^T q_i), Wuv_i transposed
+        self.w_uk = tensors[n["uk"]].view(self.heads, self.dim, self.kv_rank).contiguous()
+        self.w_uv = tensors[n["uv"]].view(self.heads, self.vdim, self.kv_rank).transpose(1, 2).contiguous()
+        self.sink = tensors[n["sink"]]
+
+    def cache_request(self) -> Optional[CacheRequest]:
+        if self.cache_from is not None:
+            return None
+        return CacheRequest("kv", heads=1, head_dim=self.kv_rank, window=None, values=False, name="latent")
+
+    def forward(self, h: torch.Tensor, ctx, view, stream: Optional[torch.Tensor] = None, next_norm=None) -> torch.Tensor:
+        lib, t, dt = self.env.lib, h.shape[0], self.env.dtype
+        owns = self.cache_from is None
+        down = linear(lib, h, self.w_down, torch.float32)                     # [T, q_rank (+ kv_rank)]
+        cq = torch.empty((t, self.q_rank), dtype=dt, device=h.device)
+        lib.latent_norm_store(down, self.q_rank, self.q_gain, cq, self.kv_rank if owns else 0, self.kv_gain,
+                              view.k_pages if owns else None, ctx, view.block_table, self.eps, dt)
+        q = linear(lib, cq, self.w_uq, torch.float32)                         # [T, heads * dim]
+        ql = torch.empty((t, self.heads * self.kv_rank), dtype=dt, device=h.device)
+        lib.heads_linear(q, self.w_uk, ql)                                    # the queries in the latent's space
+        ol = torch.empty((t, self.heads * self.kv_rank), dtype=dt, device=h.device)
+        lib.attention_sinks(ql.view(t, self.heads, self.kv_rank), view.k_pages, view.k_pages, ol, ctx.tok_pos, ctx.tok_seq,
+                            view.block_table, self.heads, 1, self.kv_rank, self.scale, None, self.sink)
+        o = torch.empty((t, self.heads * self.vdim), dtype=dt, device=h.device)
+        lib.heads_linear(ol, self.w_uv, o)
+        return linear(lib, o, self.w_o, torch.float32)
+
+
+register_mixer("latent_attention", LatentAttention)

@@ -53,4 +53,45 @@ class RMSNorm(Part):
         return out
 
 
+class LayerNorm(Part):
+    """(x - mean) / sqrt(variance + eps) * weight + bias, the variance being the mean of the squared deviations;
+    all of it in float32.  Parameters: size, eps, bias (True), names ({"weight": ..., "bias": ...}: the tensors'
+    names below the part's prefix; an empty name is the prefix itself).  The stream may come in several copies
+    [S, T, E]: the norm then reads sum_s coef[s] x[s] (`coef` None: the plain sum)."""
+    graph_safe = True
+    plan_safe = True
+
+    def __init__(self, params: Dict, env: BuildEnv):
+        self.size = int(params["size"])
+        self.eps = float(params["eps"])
+        self.has_bias = bool(params.get("bias", True))
+        self.names = dict({"weight": "weight", "bias": "bias"}, **(params.get("names") or {}))
+        self.env = env
+        self.weight: Optional[torch.Tensor] = None
+        self.bias: Optional[torch.Tensor] = None
+
+    def tensor_specs(self) -> Dict[str, TensorSpec]:
+        out = {self.names["weight"]: TensorSpec((self.size,), role="gain", init="ones_normal")}
+        if self.has_bias:
+            out[self.names["bias"]] = TensorSpec((self.size,), role="gain", init="normal")
+        return out
+
+    def tensor_names(self, base: str) -> Dict[str, str]:
+        """full name -> the part's own name, for an owner that stores the norm under `base`."""
+        return {".".join(p for p in (base, name) if p): name for name in self.tensor_specs()}
+
+    def load(self, tensors: Dict[str, torch.Tensor]) -> None:
+        self.weight = tensors[self.names["weight"]]
+        self.bias = tensors[self.names["bias"]] if self.has_bias else None
+
+    def forward(self, x: torch.Tensor, delta: Optional[torch.Tensor] = None, rows: Optional[torch.Tensor] = None,
+                coef: Optional[torch.Tensor] = None, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+        t = x.shape[-2]
+        n = t if rows is None else rows.shape[0]
+        out = torch.empty((n, self.size), dtype=out_dtype or self.env.dtype, device=x.device)
+        self.env.lib.streams_layernorm(x, coef, self.weight, self.bias, self.eps, rows, out, delta=delta)
+        return out
+
+
 register_norm("rmsnorm", RMSNorm)
+register_norm("layernorm", LayerNorm)
