@@ -35,7 +35,7 @@ class TensorSpec:
     role "gain":   a norm's gain, held in float32 (widening is exact);
     role "table":  integers, held as int32.
     init names the random initialisation: "normal" is N(0, std), "ones_normal"
-    is 1 + N(0, norm_std)."""
+    is 1 + N(0, norm_std), "eye_normal" the identity matrix + N(0, norm_std)."""
     shape: Tuple[int, ...]
     role: str = "matrix"
     init: str = "normal"

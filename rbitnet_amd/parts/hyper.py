@@ -42,7 +42,7 @@ class _OwnTensors(Part):
         for p in b.sublayers:
             out[b.name("in", p)] = TensorSpec((s,), role="gain", init="ones_normal")
             out[b.name("out", p)] = TensorSpec((s,), role="gain", init="ones_normal")
-            out[b.name("mix", p)] = TensorSpec((s, s), role="gain", init="normal")
+            out[b.name("mix", p)] = TensorSpec((s, s), role="gain", init="eye_normal")
             out[b.name("scale", p)] = TensorSpec((b.hidden,), role="gain", init="ones_normal")
         if b.conv is not None:
             out[b.conv_name] = b.conv.tensor_spec()

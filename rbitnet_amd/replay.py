@@ -130,11 +130,16 @@ def main(argv: Optional[list] = None) -> int:
     ap.add_argument("--dtype", required=True, choices=["bfloat16", "float32"])
     ap.add_argument("--out", required=True, help="folder for <step>.f32 files")
     ap.add_argument("--max-tokens", type=int, required=True,
-                    help="most tokens live requests hold at any time (each rounded up to 64); sizes the cache")
+                    help="most tokens live requests hold at any time; sizes the cache")
     args = ap.parse_args(argv)
     try:
+        from .cache import PAGE_SIZE
         from .engine import Engine
-        engine = Engine.load_path(args.model, dtype=args.dtype, max_tokens=args.max_tokens)
+        # every live request holds at least one token and may leave most of its last page empty: room for that
+        # many requests (64 at most), and a page more for each than their tokens alone would take
+        slots = max(1, min(int(args.max_tokens), 64))
+        engine = Engine.load_path(args.model, dtype=args.dtype, max_tokens=int(args.max_tokens) + PAGE_SIZE * slots,
+                                  max_batch=slots)
         replay(engine, sys.stdin, args.out)
     except RbitnetError as e:
         print(f"error: {e}", file=sys.stderr)
