@@ -312,6 +312,113 @@ def stream_probe(cfg, tokens: int = 8, copies: int = 8) -> dict:
     return out
 
 
+# ---------------------------------------------------------------- another design beside its closest Llama shape
+def bagonex_config(width: int, layers: int, heads: int, dim: int, ff: int, q_rank: int, kv_rank: int, vocab: int,
+                   streams: int = 2, low_rank: int = 128) -> dict:
+    """Layers alternate between the gated delta rule and attention through a latent; every second latent layer reads
+    the latents of the one before it."""
+    out = []
+    for i in range(layers):
+        if i % 2 == 0:
+            mixer = {"heads": heads, "kv_heads": heads, "dim": dim, "vdim": dim, "conv": 4, "decay_rank": low_rank,
+                     "gate_rank": low_rank}
+            out.append({"type": "channel_delta", "mixer": mixer, "mlp": {"kind": "dense", "ff": ff}})
+        else:
+            mixer = {"heads": heads, "dim": dim, "vdim": dim, "q_rank": q_rank, "kv_rank": kv_rank, "scale": dim ** -0.5}
+            if i % 4 == 3:
+                mixer["kv_from"] = i - 2
+            out.append({"type": "latent_attention", "mixer": mixer, "mlp": {"kind": "dense", "ff": ff}})
+    return {"architecture": "Bagonex", "vocab": vocab, "width": width, "streams": streams, "norm": {"eps": 1e-6},
+            "canon": {"taps": 4}, "logit_softcap": 30.0, "layers": out}
+
+
+# size -> (the Bagonex configuration, the Llama shape of equal width, depth and feed-forward width beside it)
+DESIGN_SIZES = {
+    "w2048": (bagonex_config(2048, 16, 16, 128, 8192, 768, 128, 128256), _other(2048, 8192, 32, 8, 64, 16)),
+    "w4096": (bagonex_config(4096, 8, 32, 128, 14336, 1536, 128, 128256), dict(LLAMA3_8B, num_hidden_layers=8)),
+    "w1024": (bagonex_config(1024, 12, 8, 64, 4096, 384, 64, 32000, low_rank=64), _other(1024, 4096, 16, 4, 64, 12, vocab=32000)),
+}
+
+
+def _kernel_table(engine, run) -> dict:
+    """Per kernel wrapper: calls and mean microseconds on the GPU while `run()` executes, launch by launch."""
+    from .csrc.lib import TIMED_OPS, KernelTimes
+    lib = engine.lib
+    graphs, plans = engine.use_graphs, engine.use_plans
+    engine.use_graphs = engine.use_plans = False
+    times = KernelTimes()
+    for name in TIMED_OPS:
+        setattr(lib, name, times.wrap(name, getattr(lib, name)))
+    lib.times = times
+    try:
+        run()
+        totals = times.totals()
+    finally:
+        for name in TIMED_OPS:
+            delattr(lib, name)
+        lib.times = None
+        engine.use_graphs, engine.use_plans = graphs, plans
+    return {name: {"calls": calls, "mean_us": round(ms * 1e3 / max(1, calls), 2), "total_ms": round(ms, 3)}
+            for name, (calls, ms) in sorted(totals.items(), key=lambda kv: -kv[1][1])}
+
+
+def design_run(size: str, dtype: str, batch: int, steps: int, warmup: int, prefill_tokens: int, prompt_len: int) -> dict:
+    """Prefill and decode throughput of a Bagonex model with random weights beside the Llama shape of equal size, and
+    where each spends its time, kernel by kernel."""
+    import numpy as np
+    import torch
+    from .engine import Engine
+    out = {"size": size, "dtype": dtype, "batch": batch, "steps": steps, "prefill_tokens": prefill_tokens,
+           "prompt_len": prompt_len}
+    for label, cfg in zip(("bagonex", "llama"), DESIGN_SIZES[size]):
+        cfg = dict(cfg)
+        ctx_cap = prompt_len + steps + warmup + 64
+        if "max_position_embeddings" in cfg:
+            cfg["max_position_embeddings"] = max(cfg["max_position_embeddings"], prefill_tokens + 64, ctx_cap)
+        engine = Engine.random(cfg, seed=0, dtype="bfloat16" if dtype == "bf16" else "float32", std=0.02, norm_std=0.02,
+                               max_batch=batch, max_tokens=max(batch * ctx_cap, prefill_tokens + 64),
+                               max_seq_len=max(ctx_cap, prefill_tokens + 64))
+        _sync()
+        dt, ctx_mean = decode_run(engine, batch, steps, warmup, prompt_len=prompt_len)
+        rng = np.random.default_rng(1)
+        prompt = [int(t) for t in rng.integers(0, engine.spec.vocab_size, size=prefill_tokens)]
+
+        def prefill_once():
+            slot = engine.alloc_slot()
+            _sync()
+            t0 = time.perf_counter()
+            engine.step([(slot, prompt)], "last")
+            _sync()
+            engine.free_slot(slot)
+            return time.perf_counter() - t0
+
+        times = [prefill_once() for _ in range(PREFILL_RUNS + 1)]
+        pt = sorted(times[1:])[len(times[1:]) // 2]
+        row = {"decode_tokens_per_s": round(batch * steps / dt, 1), "decode_ms_per_step": round(dt / steps * 1e3, 4),
+               "prefill_tokens_per_s": round(prefill_tokens / pt, 1), "prefill_ms": round(pt * 1e3, 3),
+               "weight_gb": round(engine.model.weight_bytes() / 1e9, 3),
+               "decode_weight_stream_frac": round(engine.model.weight_bytes() / (dt / steps) / PEAK_HBM, 4),
+               "mean_context": round(ctx_mean, 1)}
+        row["prefill_kernels"] = _kernel_table(engine, prefill_once)
+        # eight decode steps by themselves: the prompts go in before the timers are on
+        slots = [engine.alloc_slot() for _ in range(batch)]
+        first = engine.sampler.sample(engine.step(
+            [(sl, [int(t) for t in rng.integers(0, engine.spec.vocab_size, size=prompt_len)]) for sl in slots], "last"))
+        state = {"tokens": first}
+
+        def eight_steps():
+            for _ in range(8):
+                state["tokens"] = engine.decode_step(slots, state["tokens"])
+
+        row["decode_kernels"] = _kernel_table(engine, eight_steps)
+        for sl in slots:
+            engine.free_slot(sl)
+        out[label] = row
+        del engine
+        torch.cuda.empty_cache()
+    return out
+
+
 def main(argv=None) -> int:
     ap = argparse.ArgumentParser(prog="bench")
     ap.add_argument("--gpus", type=int, default=1)
@@ -341,6 +448,9 @@ def main(argv=None) -> int:
     ap.add_argument("--stream-probe", action="store_true",
                     help="no benchmark line: the named shape's decode products of 8 tokens beside a kernel that only "
                          "reads as many bytes")
+    ap.add_argument("--design", default="", metavar="SIZE",
+                    help=f"no benchmark line: a Bagonex model of this size ({', '.join(sorted(DESIGN_SIZES))}) beside the Llama "
+                         "shape of equal width, depth and feed-forward width: prefill and decode throughput, and the time per kernel")
     ap.add_argument("--tokens", default="1,8,64,512,2048", help="token counts of --planner-sweep")
     ap.add_argument("--sweep-detail", default=None, help="--planner-sweep: a file for every candidate's time")
     ap.add_argument("--prefill-tokens", type=int, default=PREFILL_TOKENS,
@@ -352,6 +462,12 @@ def main(argv=None) -> int:
         print(f"bench.py measures one GPU only (this library has no multi-GPU path); --gpus {args.gpus} is not run")
         return 2
 
+    if args.design:
+        if args.design not in DESIGN_SIZES:
+            ap.error(f"unknown --design {args.design!r}; one of {', '.join(sorted(DESIGN_SIZES))}")
+        print(json.dumps(design_run(args.design, args.dtype, args.batch, args.steps, args.warmup, args.prefill_tokens,
+                                    int(args.prompt_len.split(",")[0]))))
+        return 0
     names = [v for v in args.model.split(",") if v]
     for name in names:
         if name not in MODELS:

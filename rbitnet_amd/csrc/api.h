@@ -125,6 +125,16 @@ int rb_attention_generic_sinks(const void* q, const void* k_pages, const void* v
                                int bt_stride, int n_tokens, int n_heads, int n_kv_heads, int head_dim, float scale,
                                int window, const float* sinks, void* stream);
 
+// The matrix-core kernels with sinks as above (float32 [Hq] or null); v_pages may be k_pages.
+int rb_attention_prefill_bf16_sinks(const void* q, const void* k_pages, const void* v_pages, void* out,
+                                    const int32_t* cu_seqlens, const int32_t* past_len, const int32_t* block_table,
+                                    int bt_stride, int n_seqs, int max_q_len, int n_heads, int n_kv_heads, int head_dim,
+                                    float scale, int window, const float* sinks, void* stream);
+int rb_attention_decode_bf16_sinks(const void* q, const void* k_pages, const void* v_pages, void* out,
+                                   const int32_t* tok_pos, const int32_t* block_table, int bt_stride, int n_seqs,
+                                   int n_heads, int n_kv_heads, int head_dim, float scale, int window, int n_splits,
+                                   float* workspace, const float* sinks, void* stream);
+
 // ---- a residual stream in several copies, layer norm, xIELU, the cap of logits (streams.hip)
 // x [S, T, E] float32, stream_stride floats from one copy to the next.
 //   rb_embed_streams:     x[s][t, :] = table[ids[t], :] for every copy
@@ -147,12 +157,10 @@ int rb_tanh_cap(float* x, float cap, long long n, void* stream);
 // ---- layers with a fixed-size state per sequence (recurrent.hip)
 // Causal convolution over time per channel: y[t, c] = (residual ? x[t, c] : 0) + sum_d w[c, taps-1-d] x[t-d, c], act 1: silu.
 // x float32 rows x_stride apart; rows before the step come from state [slots, taps-1, C] (the sequence's last taps-1
-// inputs, oldest first; zero for a fresh slot).  rb_short_conv_state, afterwards, moves the state on by the step's rows.
-int rb_short_conv(const float* x, long long x_stride, const float* w, int taps, const float* state, const int32_t* tok_pos,
-                  const int32_t* tok_seq, const int32_t* past_len, const int32_t* slots, void* out, long long out_stride,
-                  int out_dtype, int residual, int act, int n_tokens, int channels, void* stream);
-int rb_short_conv_state(const float* x, long long x_stride, int taps, float* state, const int32_t* cu_seqlens,
-                        const int32_t* slots, int n_seqs, int channels, void* stream);
+// inputs, oldest first; zero for a fresh slot), which the same launch then moves on by the step's rows.
+int rb_short_conv(const float* x, long long x_stride, const float* w, int taps, float* state, const int32_t* tok_pos,
+                  const int32_t* tok_seq, const int32_t* cu_seqlens, const int32_t* slots, void* out, long long out_stride,
+                  int out_dtype, int residual, int act, int n_tokens, int n_seqs, int channels, void* stream);
 // What enters the gated delta rule, in place: qk [T, qk_stride] holds Hk q heads, then Hk k heads, of `dim` numbers;
 // each becomes x / sqrt(sum x^2 + unit_eps), q times q_scale.  a [T, H, dim] (rows a_stride apart) becomes the decay
 // exp(-exp(a_log[h]) softplus(a + dt_bias)); beta [T, H] = sigmoid(b_in[t * b_stride + h]).

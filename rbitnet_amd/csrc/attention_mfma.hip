@@ -29,7 +29,7 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void attn_prefill_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_pages, const bf16_t* __restrict__ v_pages,
     bf16_t* __restrict__ out, const int32_t* __restrict__ cu_seqlens, const int32_t* __restrict__ past_len,
     const int32_t* __restrict__ block_table, int bt_stride, int n_heads, int n_kv, float scale_log2, int window,
-    int gw, int paired) {
+    int gw, int paired, const float* __restrict__ sinks) {
   constexpr int KLD = D + 8;          // K tile row: D + 8 elements, rows 16 bytes apart in bank space
   constexpr int VLD = RB_PAGE + 8;    // V^T tile row: 64 keys + 8
   constexpr int DC = D / 8;           // 16-byte chunks per row
@@ -285,6 +285,8 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void attn_prefill_kernel(
   }
 
   if (!wave_on || !q_ok) return;
+  // a sink: a term of the denominator with no key and no value, not scaled (m_run is in the exponent's base-2 units)
+  if (sinks) l_run += __builtin_amdgcn_exp2f(fmaf(sinks[head], LOG2E, -m_run));
   const float inv = l_run > 0.f ? 1.0f / l_run : 0.f;
   bf16_t* orow = out + ((size_t)(seq_start + ql) * n_heads + head) * D;
 #pragma unroll
@@ -307,8 +309,17 @@ extern "C" int rb_attention_prefill_bf16(const void* q, const void* k_pages, con
                                          const int32_t* block_table, int bt_stride, int n_seqs, int max_q_len,
                                          int n_heads, int n_kv_heads, int head_dim, float scale, int window,
                                          void* stream) {
-  RB_RECORDED(rb_attention_prefill_bf16(q, k_pages, v_pages, out, cu_seqlens, past_len, block_table, bt_stride, n_seqs,
-                                        max_q_len, n_heads, n_kv_heads, head_dim, scale, window, stream));
+  return rb_attention_prefill_bf16_sinks(q, k_pages, v_pages, out, cu_seqlens, past_len, block_table, bt_stride, n_seqs,
+                                         max_q_len, n_heads, n_kv_heads, head_dim, scale, window, nullptr, stream);
+}
+
+extern "C" int rb_attention_prefill_bf16_sinks(const void* q, const void* k_pages, const void* v_pages, void* out,
+                                               const int32_t* cu_seqlens, const int32_t* past_len,
+                                               const int32_t* block_table, int bt_stride, int n_seqs, int max_q_len,
+                                               int n_heads, int n_kv_heads, int head_dim, float scale, int window,
+                                               const float* sinks, void* stream) {
+  RB_RECORDED(rb_attention_prefill_bf16_sinks(q, k_pages, v_pages, out, cu_seqlens, past_len, block_table, bt_stride, n_seqs,
+                                              max_q_len, n_heads, n_kv_heads, head_dim, scale, window, sinks, stream));
   RB_REQUIRE(n_seqs > 0 && max_q_len > 0, "rb_attention_prefill_bf16: empty batch");
   RB_REQUIRE(n_heads > 0 && n_kv_heads > 0 && n_heads % n_kv_heads == 0,
              "rb_attention_prefill_bf16: bad head counts Hq=%d Hk=%d", n_heads, n_kv_heads);
@@ -336,7 +347,7 @@ extern "C" int rb_attention_prefill_bf16(const void* q, const void* k_pages, con
   attn_prefill_kernel<DV, NWV><<<grid, 64 * NWV, 0, s>>>((const bf16_t*)q, (const bf16_t*)k_pages,              \
                                                          (const bf16_t*)v_pages, (bf16_t*)out, cu_seqlens,      \
                                                          past_len, block_table, bt_stride, n_heads, n_kv_heads, \
-                                                         sl2, window, gw, paired)
+                                                         sl2, window, gw, paired, sinks)
   if (head_dim == 128) {
     if (nw == 8) RB_PF(128, 8);
     else RB_PF(128, 4);
@@ -420,7 +431,8 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
     const float* __restrict__ qkv, const bf16_t* __restrict__ q_in, const float* __restrict__ cos_t,
     const float* __restrict__ sin_t, int style, bf16_t* k_pages, bf16_t* v_pages, bf16_t* __restrict__ out,
     const int32_t* __restrict__ tok_pos, const int32_t* __restrict__ block_table, int bt_stride, int n_heads,
-    int n_kv, float scale_log2, int window, int n_splits, float* __restrict__ ws, int qkv_terms, size_t qkv_stride) {
+    int n_kv, float scale_log2, int window, int n_splits, float* __restrict__ ws, int qkv_terms, size_t qkv_stride,
+    const float* __restrict__ sinks) {
   constexpr int DL = D / 64;          // output elements per lane
   constexpr int QC = D / 32;          // 16-byte chunks of a quarter row of K
   constexpr int QP = D / 8;           // bfloat16 pairs of a quarter row
@@ -616,6 +628,7 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
       l += red_l[w][gg] * f;
     }
     if (n_splits == 1) {
+      if (sinks) l += exp2f(fmaf(sinks[kvh * G + gg], LOG2E, -m_safe));      // the sink: in the denominator only
       out[((size_t)b * n_heads + kvh * G + gg) * D + d] = f32_to_bf16(l > 0.f ? a / l : 0.f);
     } else {
       float* dst = ws + (((size_t)b * n_heads + kvh * G + gg) * n_splits + split) * (D + 2);
@@ -670,7 +683,8 @@ __global__ __launch_bounds__(64 * NW) void attn_decode_mfma_kernel(
     const float* __restrict__ qkv, const bf16_t* __restrict__ q_in, const float* __restrict__ cos_t,
     const float* __restrict__ sin_t, int style, bf16_t* k_pages, bf16_t* v_pages, bf16_t* __restrict__ out,
     const int32_t* __restrict__ tok_pos, const int32_t* __restrict__ block_table, int bt_stride, int n_heads,
-    int n_kv, float scale_log2, int window, int n_splits, float* __restrict__ ws, int qkv_terms, size_t qkv_stride) {
+    int n_kv, float scale_log2, int window, int n_splits, float* __restrict__ ws, int qkv_terms, size_t qkv_stride,
+    const float* __restrict__ sinks) {
   constexpr int KS = D / 32;          // depth steps of the score product
   constexpr int DT = D / 16;          // d tiles of the output product
   constexpr int HALF = D / 2;
@@ -947,6 +961,7 @@ __global__ __launch_bounds__(64 * NW) void attn_decode_mfma_kernel(
       l += ((lw[0] + lw[16]) + (lw[32] + lw[48])) * f;
     }
     if (n_splits == 1) {
+      if (sinks) l += exp2f(fmaf(sinks[kvh * G + gg], LOG2E, -m_safe));      // the sink: in the denominator only
       out[((size_t)b * n_heads + kvh * G + gg) * D + d] = f32_to_bf16(l > 0.f ? a / l : 0.f);
     } else {
       float* dst = ws + (((size_t)b * n_heads + kvh * G + gg) * n_splits + split) * (D + 2);
@@ -960,7 +975,8 @@ __global__ __launch_bounds__(64 * NW) void attn_decode_mfma_kernel(
 }
 
 template <int D>
-__global__ void attn_decode_combine_kernel(const float* __restrict__ ws, bf16_t* __restrict__ out, int n_splits) {
+__global__ void attn_decode_combine_kernel(const float* __restrict__ ws, bf16_t* __restrict__ out, int n_splits,
+                                           const float* __restrict__ sinks, int n_heads) {
   const size_t row = blockIdx.x;            // sequence * heads + head
   const int d = threadIdx.x;
   const float* src = ws + row * n_splits * (D + 2);
@@ -973,6 +989,7 @@ __global__ void attn_decode_combine_kernel(const float* __restrict__ ws, bf16_t*
     a += src[(size_t)s * (D + 2) + d] * f;
     l += src[(size_t)s * (D + 2) + D + 1] * f;
   }
+  if (sinks) l += exp2f(fmaf(sinks[row % n_heads], LOG2E, -m_safe));          // the sink: in the denominator only
   out[row * D + d] = f32_to_bf16(l > 0.f ? a / l : 0.f);
 }
 
@@ -993,6 +1010,7 @@ struct DecodeArgs {
   float* ws;
   int qkv_terms;          // fused: qkv as so many terms to be added up, qkv_stride floats apart
   size_t qkv_stride;
+  const float* sinks;     // per query head, or null
 };
 
 template <int D, int G, bool FUSED>
@@ -1000,8 +1018,8 @@ static void launch_decode(const DecodeArgs& a, hipStream_t s) {
   dim3 grid(a.n_splits, a.n_kv, a.n_seqs);
   attn_decode_kernel<D, G, FUSED><<<grid, 256, 0, s>>>(a.qkv, a.q, a.cos_t, a.sin_t, a.style, a.k, a.v, a.out,
                                                        a.tok_pos, a.bt, a.bt_stride, a.n_heads, a.n_kv, a.sl2,
-                                                       a.window, a.n_splits, a.ws, a.qkv_terms, a.qkv_stride);
-  if (a.n_splits > 1) attn_decode_combine_kernel<D><<<a.n_seqs * a.n_heads, D, 0, s>>>(a.ws, a.out, a.n_splits);
+                                                       a.window, a.n_splits, a.ws, a.qkv_terms, a.qkv_stride, a.sinks);
+  if (a.n_splits > 1) attn_decode_combine_kernel<D><<<a.n_seqs * a.n_heads, D, 0, s>>>(a.ws, a.out, a.n_splits, a.sinks, a.n_heads);
 }
 
 template <int D, int NW, bool FUSED, int ONCE>
@@ -1018,8 +1036,8 @@ static int launch_decode_mfma_nw(const DecodeArgs& a, hipStream_t s) {
   dim3 grid(a.n_splits, a.n_kv, a.n_seqs);
   kern<<<grid, 64 * NW, lds, s>>>(a.qkv, a.q, a.cos_t, a.sin_t, a.style, a.k, a.v, a.out, a.tok_pos, a.bt,
                                   a.bt_stride, a.n_heads, a.n_kv, a.sl2, a.window, a.n_splits, a.ws, a.qkv_terms,
-                                  a.qkv_stride);
-  if (a.n_splits > 1) attn_decode_combine_kernel<D><<<a.n_seqs * a.n_heads, D, 0, s>>>(a.ws, a.out, a.n_splits);
+                                  a.qkv_stride, a.sinks);
+  if (a.n_splits > 1) attn_decode_combine_kernel<D><<<a.n_seqs * a.n_heads, D, 0, s>>>(a.ws, a.out, a.n_splits, a.sinks, a.n_heads);
   return 0;
 }
 
@@ -1098,11 +1116,20 @@ extern "C" int rb_attention_decode_bf16(const void* q, const void* k_pages, cons
                                         const int32_t* tok_pos, const int32_t* block_table, int bt_stride,
                                         int n_seqs, int n_heads, int n_kv_heads, int head_dim, float scale,
                                         int window, int n_splits, float* workspace, void* stream) {
-  RB_RECORDED(rb_attention_decode_bf16(q, k_pages, v_pages, out, tok_pos, block_table, bt_stride, n_seqs, n_heads, n_kv_heads,
-                                       head_dim, scale, window, n_splits, workspace, stream));
+  return rb_attention_decode_bf16_sinks(q, k_pages, v_pages, out, tok_pos, block_table, bt_stride, n_seqs, n_heads,
+                                        n_kv_heads, head_dim, scale, window, n_splits, workspace, nullptr, stream);
+}
+
+extern "C" int rb_attention_decode_bf16_sinks(const void* q, const void* k_pages, const void* v_pages, void* out,
+                                              const int32_t* tok_pos, const int32_t* block_table, int bt_stride,
+                                              int n_seqs, int n_heads, int n_kv_heads, int head_dim, float scale,
+                                              int window, int n_splits, float* workspace, const float* sinks,
+                                              void* stream) {
+  RB_RECORDED(rb_attention_decode_bf16_sinks(q, k_pages, v_pages, out, tok_pos, block_table, bt_stride, n_seqs, n_heads,
+                                             n_kv_heads, head_dim, scale, window, n_splits, workspace, sinks, stream));
   DecodeArgs a = {nullptr, (const bf16_t*)q, nullptr, nullptr, 0, (bf16_t*)k_pages, (bf16_t*)v_pages, (bf16_t*)out,
                   tok_pos, block_table, bt_stride, n_seqs, n_heads, n_kv_heads, scale * LOG2E, window, n_splits,
-                  workspace, 1, 0};
+                  workspace, 1, 0, sinks};
   return dispatch_decode<false>(a, head_dim, (hipStream_t)stream, "rb_attention_decode_bf16");
 }
 
@@ -1121,6 +1148,6 @@ extern "C" int rb_attention_decode_fused_bf16(const float* qkv, int qkv_terms, l
              qkv_term_stride);
   DecodeArgs a = {qkv, nullptr, cos, sin, style, (bf16_t*)k_pages, (bf16_t*)v_pages, (bf16_t*)out,
                   tok_pos, block_table, bt_stride, n_seqs, n_heads, n_kv_heads, scale * LOG2E, window, n_splits,
-                  workspace, qkv_terms, (size_t)qkv_term_stride};
+                  workspace, qkv_terms, (size_t)qkv_term_stride, nullptr};
   return dispatch_decode<true>(a, head_dim, (hipStream_t)stream, "rb_attention_decode_fused_bf16");
 }

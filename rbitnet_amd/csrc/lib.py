@@ -105,8 +105,8 @@ class KernelTimes:
         return "\n".join(lines)
 
 
-TIMED_OPS = ("embed_streams", "streams_layernorm", "streams_update", "xielu", "tanh_cap", "short_conv", "short_conv_state",
-             "delta_prep", "delta_rule", "gated_rmsnorm", "latent_norm_store", "heads_linear", "embed_gather", "add_rmsnorm", "rope_kv_write", "swiglu", "gemm_generic", "gemm_bf16", "gemm_bf16_terms",
+TIMED_OPS = ("embed_streams", "streams_layernorm", "streams_update", "xielu", "tanh_cap", "short_conv",
+             "delta_prep", "delta_rule", "gated_rmsnorm", "latent_norm_store", "heads_linear", "attention_sinks", "embed_gather", "add_rmsnorm", "rope_kv_write", "swiglu", "gemm_generic", "gemm_bf16", "gemm_bf16_terms",
              "gemm_bf16_few", "attention_generic", "attention_prefill_bf16", "attention_decode_bf16",
              "attention_decode_fused_bf16", "sample")
 
@@ -148,13 +148,14 @@ class Kernels:
             "rb_probe_read": [_P, ctypes.c_longlong, _I, _I, _P, _P],
             "rb_probe_mfma": [_I, _I, _P, _P],
             "rb_attention_generic_sinks": [_P, _P, _P, _P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _F, _I, _P, _P],
+            "rb_attention_prefill_bf16_sinks": [_P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I, _P, _P],
+            "rb_attention_decode_bf16_sinks": [_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _F, _I, _I, _P, _P, _P],
             "rb_embed_streams": [_P, _I, _P, _P, _I, _L, _I, _I, _P],
             "rb_streams_layernorm": [_P, _I, _L, _P, _P, _P, _P, _F, _P, _I, _I, _P, _I, _P],
             "rb_streams_update": [_P, _I, _L, _P, _P, _P, _P, _I, _I, _P],
             "rb_xielu": [_P, _P, _P, _I, _L, _P],
             "rb_tanh_cap": [_P, _F, _L, _P],
-            "rb_short_conv": [_P, _L, _P, _I, _P, _P, _P, _P, _P, _P, _L, _I, _I, _I, _I, _I, _P],
-            "rb_short_conv_state": [_P, _L, _I, _P, _P, _P, _I, _I, _P],
+            "rb_short_conv": [_P, _L, _P, _I, _P, _P, _P, _P, _P, _P, _L, _I, _I, _I, _I, _I, _I, _P],
             "rb_delta_prep": [_P, _L, _I, _I, _P, _L, _P, _P, _I, _P, _L, _P, _F, _F, _I, _P],
             "rb_delta_rule": [_P, _P, _L, _P, _L, _P, _L, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _P],
             "rb_gated_rmsnorm": [_P, _P, _P, _L, _F, _P, _I, _I, _I, _I, _P],
@@ -351,7 +352,7 @@ class Kernels:
                                                 int(window or 0), self._stream()))
 
     def attention_prefill_bf16(self, q, k_pages, v_pages, out, cu_seqlens, past_len, block_table, n_seqs,
-                               max_q_len, n_heads, n_kv, head_dim, scale, window) -> None:
+                               max_q_len, n_heads, n_kv, head_dim, scale, window, sinks=None) -> None:
         n = q.shape[0]
         _check(q, "q", torch.bfloat16, (n, n_heads, head_dim))
         _check(k_pages, "k_pages", torch.bfloat16)
@@ -362,13 +363,16 @@ class Kernels:
         _check(cu_seqlens, "cu_seqlens", torch.int32, (n_seqs + 1,))
         _check(past_len, "past_len", torch.int32, (n_seqs,))
         _check(block_table, "block_table", torch.int32)
-        self._ok(self._lib.rb_attention_prefill_bf16(_ptr(q), _ptr(k_pages), _ptr(v_pages), _ptr(out),
-                                                     _ptr(cu_seqlens), _ptr(past_len), _ptr(block_table),
-                                                     block_table.shape[1], n_seqs, int(max_q_len), n_heads, n_kv,
-                                                     head_dim, float(scale), int(window or 0), self._stream()))
+        if sinks is not None:
+            _check(sinks, "sinks", torch.float32, (n_heads,))
+        self._ok(self._lib.rb_attention_prefill_bf16_sinks(_ptr(q), _ptr(k_pages), _ptr(v_pages), _ptr(out),
+                                                           _ptr(cu_seqlens), _ptr(past_len), _ptr(block_table),
+                                                           block_table.shape[1], n_seqs, int(max_q_len), n_heads, n_kv,
+                                                           head_dim, float(scale), int(window or 0), _ptr(sinks),
+                                                           self._stream()))
 
     def attention_decode_bf16(self, q, k_pages, v_pages, out, tok_pos, block_table, n_heads, n_kv, head_dim,
-                              scale, window, n_splits, workspace) -> None:
+                              scale, window, n_splits, workspace, sinks=None) -> None:
         n = q.shape[0]
         _check(q, "q", torch.bfloat16, (n, n_heads, head_dim))
         _check(k_pages, "k_pages", torch.bfloat16)
@@ -381,10 +385,12 @@ class Kernels:
         _check(workspace, "workspace", torch.float32)
         if workspace.numel() < n * n_heads * n_splits * (head_dim + 2):
             raise KernelError("decode attention workspace too small")
-        self._ok(self._lib.rb_attention_decode_bf16(_ptr(q), _ptr(k_pages), _ptr(v_pages), _ptr(out), _ptr(tok_pos),
-                                                    _ptr(block_table), block_table.shape[1], n, n_heads, n_kv,
-                                                    head_dim, float(scale), int(window or 0), int(n_splits),
-                                                    _ptr(workspace), self._stream()))
+        if sinks is not None:
+            _check(sinks, "sinks", torch.float32, (n_heads,))
+        self._ok(self._lib.rb_attention_decode_bf16_sinks(_ptr(q), _ptr(k_pages), _ptr(v_pages), _ptr(out), _ptr(tok_pos),
+                                                          _ptr(block_table), block_table.shape[1], n, n_heads, n_kv,
+                                                          head_dim, float(scale), int(window or 0), int(n_splits),
+                                                          _ptr(workspace), _ptr(sinks), self._stream()))
 
     def attention_decode_fused_bf16(self, qkv, cos, sin, style, k_pages, v_pages, out, tok_pos, block_table,
                                     n_heads, n_kv, head_dim, scale, window, n_splits, workspace) -> None:
@@ -490,7 +496,7 @@ class Kernels:
     def short_conv(self, x: torch.Tensor, col0: int, channels: int, w: torch.Tensor, state: Optional[torch.Tensor], ctx,
                    out: torch.Tensor, residual: bool, act: int) -> None:
         """Columns col0 .. col0 + channels of x [T, W] float32 through the causal convolution w [channels, taps];
-        state [slots, taps - 1, channels] float32 holds every sequence's last inputs."""
+        state [slots, taps - 1, channels] float32 holds every sequence's last inputs and is moved on by the step."""
         n, width = x.shape
         taps = w.shape[1]
         _check(x, "x", torch.float32)
@@ -504,21 +510,9 @@ class Kernels:
         _check(out, "out", None, (n, channels))
         _check(ctx.tok_pos, "tok_pos", torch.int32, (n,))
         self._ok(self._lib.rb_short_conv(x.data_ptr() + 4 * col0, width, _ptr(w), taps, _ptr(state) if taps > 1 else None,
-                                         _ptr(ctx.tok_pos), _ptr(ctx.tok_seq), _ptr(ctx.past_len), _ptr(ctx.slots), _ptr(out),
-                                         channels, dtype_code(out.dtype), int(bool(residual)), int(act), n, channels,
-                                         self._stream()))
-
-    def short_conv_state(self, x: torch.Tensor, col0: int, channels: int, taps: int, state: torch.Tensor, ctx) -> None:
-        """After `short_conv`: the state moves on by the step's rows."""
-        if taps <= 1:
-            return
-        n, width = x.shape
-        _check(x, "x", torch.float32)
-        _check(state, "state", torch.float32)
-        if tuple(state.shape[1:]) != (taps - 1, channels) or col0 < 0 or col0 + channels > width:
-            raise KernelError("short_conv_state: state or columns do not fit")
-        self._ok(self._lib.rb_short_conv_state(x.data_ptr() + 4 * col0, width, taps, _ptr(state), _ptr(ctx.cu_seqlens),
-                                               _ptr(ctx.slots), ctx.n_seqs, channels, self._stream()))
+                                         _ptr(ctx.tok_pos), _ptr(ctx.tok_seq), _ptr(ctx.cu_seqlens), _ptr(ctx.slots), _ptr(out),
+                                         channels, dtype_code(out.dtype), int(bool(residual)), int(act), n, ctx.n_seqs,
+                                         channels, self._stream()))
 
     def delta_prep(self, qkv: torch.Tensor, n_kv: int, dim: int, a: torch.Tensor, dt_bias: torch.Tensor, a_log: torch.Tensor,
                    n_heads: int, b_in: torch.Tensor, b_col: int, beta: torch.Tensor, q_scale: float, unit_eps: float) -> None:

@@ -15,92 +15,84 @@ __device__ __forceinline__ float rb_softplus(float v) { return v > 20.0f ? v : l
 // y[t, c] = (residual ? x[t, c] : 0) + sum_d w[c, taps - 1 - d] * x[t - d, c], d = 0 .. taps - 1, where rows
 // before the step's first come from the sequence's state (its last taps - 1 inputs, oldest first) and rows
 // before the sequence's start are zero (the state of a fresh slot is zero).  act 1: silu on the result.
+// Afterwards the state holds the last taps - 1 inputs again.  One launch: a workgroup per token for the tokens
+// that need rows of the step only, and a workgroup per sequence that walks the step's first taps - 1 tokens with
+// the old state in registers and then writes the new state, so that whoever reads the state is also who writes it.
+#define SC_MAX_TAPS 16
 template <typename TO>
 __global__ void short_conv_kernel(const float* __restrict__ x, size_t x_stride, const float* __restrict__ w, int taps,
-                                  const float* __restrict__ state, const int32_t* __restrict__ tok_pos,
-                                  const int32_t* __restrict__ tok_seq, const int32_t* __restrict__ past_len,
+                                  float* __restrict__ state, const int32_t* __restrict__ tok_pos,
+                                  const int32_t* __restrict__ tok_seq, const int32_t* __restrict__ cu_seqlens,
                                   const int32_t* __restrict__ slots, TO* __restrict__ out, size_t out_stride,
-                                  int residual, int act, int channels) {
-  const int t = blockIdx.x;
-  const int b = tok_seq[t];
-  const int pos = tok_pos[t], past = past_len[b];
-  const float* st = state + (size_t)slots[b] * (taps - 1) * channels;
-  for (int c = blockIdx.y * blockDim.x + threadIdx.x; c < channels; c += gridDim.y * blockDim.x) {
-    const float cur = x[(size_t)t * x_stride + c];
-    float acc = residual ? cur : 0.f;
-    for (int d = 0; d < taps; ++d) {
-      const int sp = pos - d;
-      float v;
-      if (sp >= past)
-        v = d == 0 ? cur : x[(size_t)(t - d) * x_stride + c];
-      else
-        v = st[(size_t)(sp - past + taps - 1) * channels + c];
-      acc = fmaf(w[(size_t)c * taps + (taps - 1 - d)], v, acc);
+                                  int residual, int act, int channels, int n_tokens) {
+  const int keep = taps - 1;
+  if ((int)blockIdx.x < n_tokens) {
+    const int t = blockIdx.x;
+    if (t - cu_seqlens[tok_seq[t]] < keep) return;           // the sequence's workgroup takes it
+    for (int c = blockIdx.y * blockDim.x + threadIdx.x; c < channels; c += gridDim.y * blockDim.x) {
+      const float cur = x[(size_t)t * x_stride + c];
+      float acc = residual ? cur : 0.f;
+      for (int d = 0; d < taps; ++d)
+        acc = fmaf(w[(size_t)c * taps + (keep - d)], d == 0 ? cur : x[(size_t)(t - d) * x_stride + c], acc);
+      if (act == 1) acc = acc * rb_sigmoid(acc);
+      Num<TO>::store(out + (size_t)t * out_stride + c, acc);
     }
-    if (act == 1) acc = acc * rb_sigmoid(acc);
-    Num<TO>::store(out + (size_t)t * out_stride + c, acc);
+    return;
+  }
+  const int b = blockIdx.x - n_tokens;
+  const int row0 = cu_seqlens[b], n = cu_seqlens[b + 1] - row0;
+  float* st = state + (size_t)slots[b] * keep * channels;
+  const int first = n < keep ? n : keep;
+  for (int c = blockIdx.y * blockDim.x + threadIdx.x; c < channels; c += gridDim.y * blockDim.x) {
+    float win[SC_MAX_TAPS], wt[SC_MAX_TAPS];                 // the last `keep` inputs, oldest first; their weights
+#pragma unroll
+    for (int j = 0; j < SC_MAX_TAPS; ++j) {
+      win[j] = j < keep ? st[(size_t)j * channels + c] : 0.f;
+      wt[j] = j < keep ? w[(size_t)c * taps + j] : 0.f;
+    }
+    const float w_cur = w[(size_t)c * taps + keep];
+    for (int i = 0; i < first; ++i) {
+      const float cur = x[(size_t)(row0 + i) * x_stride + c];
+      float acc = residual ? cur : 0.f;
+      acc = fmaf(w_cur, cur, acc);
+#pragma unroll
+      for (int j = 0; j < SC_MAX_TAPS; ++j) acc = fmaf(wt[j], win[j], acc);
+#pragma unroll
+      for (int j = 0; j < SC_MAX_TAPS - 1; ++j) win[j] = j + 1 < keep ? win[j + 1] : win[j];
+#pragma unroll
+      for (int j = 0; j < SC_MAX_TAPS; ++j)
+        if (j == keep - 1) win[j] = cur;
+      if (act == 1) acc = acc * rb_sigmoid(acc);
+      Num<TO>::store(out + (size_t)(row0 + i) * out_stride + c, acc);
+    }
+#pragma unroll
+    for (int j = 0; j < SC_MAX_TAPS; ++j)
+      if (j < keep) st[(size_t)j * channels + c] = n > keep ? x[(size_t)(row0 + n - keep + j) * x_stride + c] : win[j];
   }
 }
 
-extern "C" int rb_short_conv(const float* x, long long x_stride, const float* w, int taps, const float* state,
-                             const int32_t* tok_pos, const int32_t* tok_seq, const int32_t* past_len,
+extern "C" int rb_short_conv(const float* x, long long x_stride, const float* w, int taps, float* state,
+                             const int32_t* tok_pos, const int32_t* tok_seq, const int32_t* cu_seqlens,
                              const int32_t* slots, void* out, long long out_stride, int out_dtype, int residual,
-                             int act, int n_tokens, int channels, void* stream) {
-  RB_RECORDED(rb_short_conv(x, x_stride, w, taps, state, tok_pos, tok_seq, past_len, slots, out, out_stride, out_dtype,
-                            residual, act, n_tokens, channels, stream));
-  RB_REQUIRE(n_tokens >= 0 && channels > 0 && taps >= 1, "rb_short_conv: bad sizes T=%d C=%d taps=%d", n_tokens, channels, taps);
+                             int act, int n_tokens, int n_seqs, int channels, void* stream) {
+  RB_RECORDED(rb_short_conv(x, x_stride, w, taps, state, tok_pos, tok_seq, cu_seqlens, slots, out, out_stride, out_dtype,
+                            residual, act, n_tokens, n_seqs, channels, stream));
+  RB_REQUIRE(n_tokens >= 0 && n_seqs >= 0 && channels > 0 && taps >= 1 && taps - 1 <= SC_MAX_TAPS,
+             "rb_short_conv: bad sizes T=%d B=%d C=%d taps=%d (at most %d)", n_tokens, n_seqs, channels, taps, SC_MAX_TAPS + 1);
   RB_REQUIRE(x_stride >= channels && out_stride >= channels, "rb_short_conv: a row stride is shorter than the channels");
   RB_REQUIRE(taps == 1 || state != nullptr, "rb_short_conv: %d taps need a state", taps);
   RB_REQUIRE(act == 0 || act == 1, "rb_short_conv: unknown activation %d", act);
   if (n_tokens == 0) return 0;
-  dim3 grid(n_tokens, (channels + 255) / 256 < 16 ? (channels + 255) / 256 : 16);
+  dim3 grid(n_tokens + (taps > 1 ? n_seqs : 0), (channels + 255) / 256 < 16 ? (channels + 255) / 256 : 16);
   hipStream_t s = (hipStream_t)stream;
   if (out_dtype == RB_F32)
-    short_conv_kernel<float><<<grid, 256, 0, s>>>(x, (size_t)x_stride, w, taps, state, tok_pos, tok_seq, past_len, slots,
-                                                  (float*)out, (size_t)out_stride, residual, act, channels);
+    short_conv_kernel<float><<<grid, 256, 0, s>>>(x, (size_t)x_stride, w, taps, state, tok_pos, tok_seq, cu_seqlens, slots,
+                                                  (float*)out, (size_t)out_stride, residual, act, channels, n_tokens);
   else if (out_dtype == RB_BF16)
-    short_conv_kernel<bf16_t><<<grid, 256, 0, s>>>(x, (size_t)x_stride, w, taps, state, tok_pos, tok_seq, past_len, slots,
-                                                   (bf16_t*)out, (size_t)out_stride, residual, act, channels);
+    short_conv_kernel<bf16_t><<<grid, 256, 0, s>>>(x, (size_t)x_stride, w, taps, state, tok_pos, tok_seq, cu_seqlens, slots,
+                                                   (bf16_t*)out, (size_t)out_stride, residual, act, channels, n_tokens);
   else
     RB_REQUIRE(false, "rb_short_conv: unknown dtype %d", out_dtype);
-  RB_LAUNCH_CHECK();
-  return 0;
-}
-
-// After the step: the state becomes the last taps - 1 inputs of the sequence, oldest first.  A thread owns a
-// channel of a sequence and reads all it needs before it writes.
-#define SC_MAX_TAPS 16
-__global__ void short_conv_state_kernel(const float* __restrict__ x, size_t x_stride, int taps, float* __restrict__ state,
-                                        const int32_t* __restrict__ cu_seqlens, const int32_t* __restrict__ slots,
-                                        int channels) {
-  const int b = blockIdx.x;
-  const int row0 = cu_seqlens[b], n = cu_seqlens[b + 1] - row0;
-  const int keep = taps - 1;
-  float* st = state + (size_t)slots[b] * keep * channels;
-  for (int c = blockIdx.y * blockDim.x + threadIdx.x; c < channels; c += gridDim.y * blockDim.x) {
-    float v[SC_MAX_TAPS];
-#pragma unroll
-    for (int i = 0; i < SC_MAX_TAPS; ++i) {
-      if (i < keep) {
-        const int r = n - keep + i;          // row of the step that lands in entry i; negative: an older input
-        v[i] = r >= 0 ? x[(size_t)(row0 + r) * x_stride + c] : st[(size_t)(i + n) * channels + c];
-      }
-    }
-#pragma unroll
-    for (int i = 0; i < SC_MAX_TAPS; ++i)
-      if (i < keep) st[(size_t)i * channels + c] = v[i];
-  }
-}
-
-extern "C" int rb_short_conv_state(const float* x, long long x_stride, int taps, float* state, const int32_t* cu_seqlens,
-                                   const int32_t* slots, int n_seqs, int channels, void* stream) {
-  RB_RECORDED(rb_short_conv_state(x, x_stride, taps, state, cu_seqlens, slots, n_seqs, channels, stream));
-  RB_REQUIRE(n_seqs >= 0 && channels > 0 && taps >= 1 && taps - 1 <= SC_MAX_TAPS,
-             "rb_short_conv_state: bad sizes B=%d C=%d taps=%d (at most %d)", n_seqs, channels, taps, SC_MAX_TAPS + 1);
-  RB_REQUIRE(x_stride >= channels, "rb_short_conv_state: the row stride is shorter than the channels");
-  if (n_seqs == 0 || taps == 1) return 0;
-  dim3 grid(n_seqs, (channels + 255) / 256 < 64 ? (channels + 255) / 256 : 64);
-  short_conv_state_kernel<<<grid, 256, 0, (hipStream_t)stream>>>(x, (size_t)x_stride, taps, state, cu_seqlens, slots, channels);
   RB_LAUNCH_CHECK();
   return 0;
 }
@@ -151,10 +143,12 @@ extern "C" int rb_delta_prep(float* qk, long long qk_stride, int n_kv_heads, int
 // Per sequence and head, token after token:
 //   S <- diag(g) S;  u = beta (v - S^T k);  S <- S + k u^T;  o = S^T q
 // The columns of S (one per value channel) do not meet: a column is held by RG lanes, each with DKL of its rows in
-// registers; the two dot products over the rows are finished by shuffles among the RG lanes.  A wave holds 64 / RG
-// columns; q, k and g of a few tokens are staged in LDS for all lanes.  The state is read once and written once.
-#define DR_CHUNK 8
-template <int DKL, int RG>
+// registers; the two dot products over the rows are finished by shuffles among the RG lanes.  A workgroup is one wave
+// and holds 64 / RG columns.  Tokens go by in chunks of CH: q, k, g, v and beta of a chunk lie in LDS for all lanes, and
+// the next chunk's loads are in flight (in registers) while the current one is computed, so that a token costs its
+// arithmetic and no trip to memory; the chunk's outputs leave through LDS as whole rows.  The state is read once and
+// written once.
+template <int DKL, int RG, int CH>
 __global__ __launch_bounds__(RB_WAVE) void delta_rule_kernel(
     const float* __restrict__ q, const float* __restrict__ k, size_t qk_stride, const float* __restrict__ v,
     size_t v_stride, const float* __restrict__ g, size_t g_stride, const float* __restrict__ beta, float* __restrict__ state,
@@ -162,10 +156,13 @@ __global__ __launch_bounds__(RB_WAVE) void delta_rule_kernel(
     int n_kv, int dim, int vdim) {
   constexpr int COLS = RB_WAVE / RG;
   constexpr int DK = DKL * RG;               // rows held, >= dim; rows beyond dim stay zero
-  __shared__ float sq[DR_CHUNK][DK], sk[DR_CHUNK][DK], sg[DR_CHUNK][DK];
+  constexpr int NQ = DK * CH / RB_WAVE;      // q (or k, or g) values of a chunk per lane
+  constexpr int NV = (COLS * CH + RB_WAVE - 1) / RB_WAVE;
+  __shared__ float sq[CH][DK], sk[CH][DK], sg[CH][DK], sv[CH][COLS], so[CH][COLS], sb[CH];
   const int b = blockIdx.x, h = blockIdx.y;
   const int lane = threadIdx.x;
-  const int col = blockIdx.z * COLS + lane / RG;
+  const int col0 = blockIdx.z * COLS;
+  const int col = col0 + lane / RG;
   const int rg = lane % RG;
   const bool on = col < vdim;
   const int kvh = h / (n_heads / n_kv);
@@ -177,22 +174,47 @@ __global__ __launch_bounds__(RB_WAVE) void delta_rule_kernel(
     const int r = rg * DKL + i;
     s[i] = (on && r < dim) ? S[(size_t)r * vdim + col] : 0.f;
   }
-  for (int t0 = 0; t0 < n; t0 += DR_CHUNK) {
-    const int nt = n - t0 < DR_CHUNK ? n - t0 : DR_CHUNK;
-    __builtin_amdgcn_s_barrier();
-    for (int idx = lane; idx < nt * DK; idx += RB_WAVE) {
-      const int tt = idx / DK, i = idx - tt * DK;
+  float rq[NQ], rk[NQ], rgt[NQ], rv[NV], rb = 0.f;
+  auto fetch = [&](int t0) {
+    const int nt = n - t0 < CH ? n - t0 : CH;
+#pragma unroll
+    for (int j = 0; j < NQ; ++j) {
+      const int e = lane + RB_WAVE * j, tt = e / DK, i = e - tt * DK;
+      const bool in = tt < nt && i < dim;
       const size_t t = (size_t)(row0 + t0 + tt);
-      const bool in = i < dim;
-      sq[tt][i] = in ? q[t * qk_stride + (size_t)kvh * dim + i] : 0.f;
-      sk[tt][i] = in ? k[t * qk_stride + (size_t)kvh * dim + i] : 0.f;
-      sg[tt][i] = in ? g[t * g_stride + (size_t)h * dim + i] : 0.f;
+      rq[j] = in ? q[t * qk_stride + (size_t)kvh * dim + i] : 0.f;
+      rk[j] = in ? k[t * qk_stride + (size_t)kvh * dim + i] : 0.f;
+      rgt[j] = in ? g[t * g_stride + (size_t)h * dim + i] : 0.f;
     }
-    __builtin_amdgcn_s_barrier();
+#pragma unroll
+    for (int j = 0; j < NV; ++j) {
+      const int e = lane + RB_WAVE * j, tt = e / COLS, c = e - tt * COLS;
+      rv[j] = (tt < nt && col0 + c < vdim) ? v[(size_t)(row0 + t0 + tt) * v_stride + (size_t)h * vdim + col0 + c] : 0.f;
+    }
+    rb = lane < nt ? beta[(size_t)(row0 + t0 + lane) * n_heads + h] : 0.f;
+  };
+  if (n > 0) fetch(0);
+  for (int t0 = 0; t0 < n; t0 += CH) {
+    const int nt = n - t0 < CH ? n - t0 : CH;
+    __syncthreads();                                   // the chunk before has been read and its outputs are out
+#pragma unroll
+    for (int j = 0; j < NQ; ++j) {
+      const int e = lane + RB_WAVE * j, tt = e / DK, i = e - tt * DK;
+      sq[tt][i] = rq[j];
+      sk[tt][i] = rk[j];
+      sg[tt][i] = rgt[j];
+    }
+#pragma unroll
+    for (int j = 0; j < NV; ++j) {
+      const int e = lane + RB_WAVE * j;
+      if (e < COLS * CH) sv[e / COLS][e % COLS] = rv[j];
+    }
+    if (lane < CH) sb[lane] = rb;
+    __syncthreads();
+    if (t0 + CH < n) fetch(t0 + CH);                   // in flight while this chunk is computed
     for (int tt = 0; tt < nt; ++tt) {
-      const size_t t = (size_t)(row0 + t0 + tt);
-      const float vv = on ? v[t * v_stride + (size_t)h * vdim + col] : 0.f;
-      const float bt = beta[t * n_heads + h];
+      const float vv = sv[tt][lane / RG];
+      const float bt = sb[tt];
       float kv = 0.f;
 #pragma unroll
       for (int i = 0; i < DKL; ++i) {
@@ -210,7 +232,12 @@ __global__ __launch_bounds__(RB_WAVE) void delta_rule_kernel(
       }
 #pragma unroll
       for (int o = 1; o < RG; o <<= 1) oq += __shfl_xor(oq, o, RB_WAVE);
-      if (on && rg == 0) out[(t * n_heads + h) * vdim + col] = oq;
+      if (rg == 0) so[tt][lane / RG] = oq;
+    }
+    __syncthreads();
+    for (int e = lane; e < nt * COLS; e += RB_WAVE) {
+      const int tt = e / COLS, c = e - tt * COLS;
+      if (col0 + c < vdim) out[((size_t)(row0 + t0 + tt) * n_heads + h) * vdim + col0 + c] = so[tt][c];
     }
   }
 #pragma unroll
@@ -220,15 +247,16 @@ __global__ __launch_bounds__(RB_WAVE) void delta_rule_kernel(
   }
 }
 
-template <int DKL, int RG>
+template <int DKL, int RG, int CH>
 static void launch_delta_rule(const float* q, const float* k, size_t qk_stride, const float* v, size_t v_stride,
                               const float* g, size_t g_stride, const float* beta, float* state, const int32_t* cu_seqlens,
                               const int32_t* slots, float* out, int n_seqs, int n_heads, int n_kv, int dim, int vdim,
                               hipStream_t s) {
   constexpr int COLS = RB_WAVE / RG;
+  static_assert((DKL * RG * CH) % RB_WAVE == 0 && CH <= RB_WAVE, "a chunk's values are dealt evenly to the lanes");
   dim3 grid(n_seqs, n_heads, (vdim + COLS - 1) / COLS);
-  delta_rule_kernel<DKL, RG><<<grid, RB_WAVE, 0, s>>>(q, k, qk_stride, v, v_stride, g, g_stride, beta, state, cu_seqlens, slots,
-                                                      out, n_heads, n_kv, dim, vdim);
+  delta_rule_kernel<DKL, RG, CH><<<grid, RB_WAVE, 0, s>>>(q, k, qk_stride, v, v_stride, g, g_stride, beta, state, cu_seqlens,
+                                                          slots, out, n_heads, n_kv, dim, vdim);
 }
 
 extern "C" int rb_delta_rule(const float* q, const float* k, long long qk_stride, const float* v, long long v_stride,
@@ -245,21 +273,22 @@ extern "C" int rb_delta_rule(const float* q, const float* k, long long qk_stride
   if (n_seqs == 0) return 0;
   hipStream_t s = (hipStream_t)stream;
   const size_t qs = (size_t)qk_stride, vs = (size_t)v_stride;
-#define DR_GO(DKL, RG) \
-  launch_delta_rule<DKL, RG>(q, k, qs, v, vs, g, (size_t)g_stride, beta, state, cu_seqlens, slots, out, n_seqs, n_heads, n_kv_heads, dim, vdim, s)
-  // rows of a column over RG lanes: short chains per token, and enough waves for the GPU while sequences are few
+#define DR_GO(DKL, RG, CH) \
+  launch_delta_rule<DKL, RG, CH>(q, k, qs, v, vs, g, (size_t)g_stride, beta, state, cu_seqlens, slots, out, n_seqs, n_heads, n_kv_heads, dim, vdim, s)
+  // rows of a column over RG lanes: short chains per token, and enough waves for the GPU while sequences are few;
+  // chunks as long as the registers that hold the next one allow
   if (dim <= 16)
-    DR_GO(4, 4);
+    DR_GO(4, 4, 16);
   else if (dim <= 32)
-    DR_GO(8, 4);
+    DR_GO(8, 4, 16);
   else if (dim <= 64)
-    DR_GO(8, 8);
+    DR_GO(8, 8, 16);
   else if (dim <= 128)
-    DR_GO(16, 8);
+    DR_GO(16, 8, 16);
   else if (dim <= 256)
-    DR_GO(16, 16);
+    DR_GO(16, 16, 8);
   else
-    DR_GO(32, 16);
+    DR_GO(32, 16, 4);
 #undef DR_GO
   RB_LAUNCH_CHECK();
   return 0;

@@ -29,6 +29,8 @@ from .linear import linear, pack_rows
 DEFAULT_NAMES = {"dq": "dq", "dq_norm": "dq.norm", "uq": "uq", "dkv": "dkv", "dkv_norm": "dkv.norm", "uk": "uk", "uv": "uv",
                  "sink": "sink", "o": "o"}
 MAX_RANK = 256             # the attention kernel's largest head size
+_MATRIX_CORE_RANKS = (64, 128)     # latents of these sizes in bfloat16 go through the matrix-core attention kernels
+_DECODE_MAX_HEADS = 16             # query heads on one key/value head that the matrix-core decode kernel takes
 
 
 class LatentAttention(Part):
@@ -97,8 +99,18 @@ class LatentAttention(Part):
         ql = torch.empty((t, self.heads * self.kv_rank), dtype=dt, device=h.device)
         lib.heads_linear(q, self.w_uk, ql)                                    # the queries in the latent's space
         ol = torch.empty((t, self.heads * self.kv_rank), dtype=dt, device=h.device)
-        lib.attention_sinks(ql.view(t, self.heads, self.kv_rank), view.k_pages, view.k_pages, ol, ctx.tok_pos, ctx.tok_seq,
-                            view.block_table, self.heads, 1, self.kv_rank, self.scale, None, self.sink)
+        q3, pages, r = ql.view(t, self.heads, self.kv_rank), view.k_pages, self.kv_rank
+        fast = dt == torch.bfloat16 and r in _MATRIX_CORE_RANKS and not getattr(self.env, "generic_only", False)
+        if fast and ctx.max_q_len == 1 and self.heads <= _DECODE_MAX_HEADS:
+            n_splits, workspace = ctx.decode_workspace(self.heads, r, 1)
+            lib.attention_decode_bf16(q3, pages, pages, ol, ctx.tok_pos, view.block_table, self.heads, 1, r, self.scale, None,
+                                      n_splits, workspace, sinks=self.sink)
+        elif fast:
+            lib.attention_prefill_bf16(q3, pages, pages, ol, ctx.cu_seqlens, ctx.past_len, view.block_table, ctx.n_seqs,
+                                       ctx.max_q_len, self.heads, 1, r, self.scale, None, sinks=self.sink)
+        else:
+            lib.attention_sinks(q3, pages, pages, ol, ctx.tok_pos, ctx.tok_seq, view.block_table, self.heads, 1, r,
+                                self.scale, None, self.sink)
         o = torch.empty((t, self.heads * self.vdim), dtype=dt, device=h.device)
         lib.heads_linear(ol, self.w_uv, o)
         return linear(lib, o, self.w_o, torch.float32)

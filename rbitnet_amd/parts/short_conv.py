@@ -47,5 +47,4 @@ class ShortConv:
         lib = self.env.lib
         out = torch.empty((x.shape[0], self.channels), dtype=out_dtype, device=x.device)
         lib.short_conv(x, col0, self.channels, self.weight, state, ctx, out, self.residual, self.act)
-        lib.short_conv_state(x, col0, self.channels, self.taps, state, ctx)
         return out
