@@ -147,6 +147,10 @@ int rb_embed_streams(const void* table, int table_dtype, const int32_t* ids, flo
 int rb_streams_layernorm(float* x, int n_streams, long long stream_stride, const float* coef, const float* delta,
                          const float* weight, const float* bias, float eps, const int32_t* rows, int n_rows, int width,
                          void* out, int out_dtype, void* stream);
+int rb_streams_update_layernorm(float* x, int n_streams, long long stream_stride, const float* mix, const float* out_coef,
+                                const float* y, const float* scale, const float* coef, const float* delta, const float* weight,
+                                const float* bias, float eps, const int32_t* rows, int n_rows, int width, void* out,
+                                int out_dtype, void* stream);      // rb_streams_update (mix null: none), then the norm, in one pass
 int rb_streams_update(float* x, int n_streams, long long stream_stride, const float* mix, const float* out_coef, const float* y,
                       const float* scale, int n_tokens, int width, void* stream);
 // out = z > 0 ? softplus(act[0]) z^2 + z/2 : (1/2 + softplus(act[1])) (exp(z) - 1 - z) + z/2

@@ -64,58 +64,72 @@ extern "C" int rb_latent_norm_store(const float* proj, long long stride, int q_r
 
 // ---------------------------------------------------------------- a product per head
 // y[t, h, n] = sum_k w[h, k, n] * x[t, h, k]: H small matrices, stored [H, K, N] (the output index runs fastest, so
-// that neighbouring lanes read neighbouring weights).  A wave takes HL_TOKENS tokens and 64 output columns of one
-// head: the tokens' inputs in LDS, a lane per column with one sum per token, eight weights in flight per lane.
+// that neighbouring lanes read neighbouring weights).  A workgroup of four waves takes HL_TOKENS tokens and 64 output
+// columns of one head: the tokens' inputs in LDS, a lane per column with one sum per token; the waves share the inner
+// index (wave w takes k = w, w + 4, ...), sixteen weights in flight per lane, and add up through LDS in a fixed order.
 #define HL_TOKENS 16
+#define HL_WAVES 4
 template <typename TX, typename TW, typename TY>
-__global__ __launch_bounds__(RB_WAVE) void heads_linear_kernel(const TX* __restrict__ x, const TW* __restrict__ w,
-                                                               TY* __restrict__ y, int n_tokens, int n_heads, int n, int k) {
-  extern __shared__ float xs[];                  // [HL_TOKENS][k]
+__global__ __launch_bounds__(RB_WAVE * HL_WAVES) void heads_linear_kernel(const TX* __restrict__ x, const TW* __restrict__ w,
+                                                                          TY* __restrict__ y, int n_tokens, int n_heads, int n, int k) {
+  extern __shared__ float xs[];                  // [HL_TOKENS][k], then [HL_WAVES - 1][HL_TOKENS][64] partial sums
+  float* part = xs + HL_TOKENS * k;
   const int t0 = blockIdx.x * HL_TOKENS, h = blockIdx.y;
+  const int lane = threadIdx.x & (RB_WAVE - 1), wave = threadIdx.x / RB_WAVE;
   const int nt = n_tokens - t0 < HL_TOKENS ? n_tokens - t0 : HL_TOKENS;
-  for (int idx = threadIdx.x; idx < HL_TOKENS * k; idx += RB_WAVE) {
+  for (int idx = threadIdx.x; idx < HL_TOKENS * k; idx += RB_WAVE * HL_WAVES) {
     const int tt = idx / k, kk = idx - tt * k;
     xs[idx] = tt < nt ? Num<TX>::load(x + ((size_t)(t0 + tt) * n_heads + h) * k + kk) : 0.f;
   }
   __syncthreads();
-  const int col = blockIdx.z * RB_WAVE + threadIdx.x;
-  if (col >= n) return;
-  const TW* wh = w + (size_t)h * k * n + col;
+  const int col = blockIdx.z * RB_WAVE + lane;
+  const bool on = col < n;
+  const TW* wh = w + (size_t)h * k * n + (on ? col : 0);
   float acc[HL_TOKENS];
 #pragma unroll
   for (int tt = 0; tt < HL_TOKENS; ++tt) acc[tt] = 0.f;
-  int kk = 0;
-  for (; kk + 8 <= k; kk += 8) {
-    float wv[8];
+  int kk = wave;
+  for (; kk + 15 * HL_WAVES < k; kk += 16 * HL_WAVES) {
+    float wv[16];
 #pragma unroll
-    for (int j = 0; j < 8; ++j) wv[j] = Num<TW>::load(wh + (size_t)(kk + j) * n);
+    for (int j = 0; j < 16; ++j) wv[j] = Num<TW>::load(wh + (size_t)(kk + j * HL_WAVES) * n);
 #pragma unroll
-    for (int j = 0; j < 8; ++j)
+    for (int j = 0; j < 16; ++j)
 #pragma unroll
-      for (int tt = 0; tt < HL_TOKENS; ++tt) acc[tt] = fmaf(wv[j], xs[tt * k + kk + j], acc[tt]);
+      for (int tt = 0; tt < HL_TOKENS; ++tt) acc[tt] = fmaf(wv[j], xs[tt * k + kk + j * HL_WAVES], acc[tt]);
   }
-  for (; kk < k; ++kk) {
+  for (; kk < k; kk += HL_WAVES) {
     const float wv = Num<TW>::load(wh + (size_t)kk * n);
 #pragma unroll
     for (int tt = 0; tt < HL_TOKENS; ++tt) acc[tt] = fmaf(wv, xs[tt * k + kk], acc[tt]);
   }
+  if (wave > 0) {
 #pragma unroll
-  for (int tt = 0; tt < HL_TOKENS; ++tt)
-    if (tt < nt) Num<TY>::store(y + ((size_t)(t0 + tt) * n_heads + h) * n + col, acc[tt]);
+    for (int tt = 0; tt < HL_TOKENS; ++tt) part[((wave - 1) * HL_TOKENS + tt) * RB_WAVE + lane] = acc[tt];
+  }
+  __syncthreads();
+  if (wave > 0 || !on) return;
+#pragma unroll
+  for (int tt = 0; tt < HL_TOKENS; ++tt) {
+    float v = acc[tt];
+#pragma unroll
+    for (int ww = 0; ww < HL_WAVES - 1; ++ww) v += part[(ww * HL_TOKENS + tt) * RB_WAVE + lane];
+    if (tt < nt) Num<TY>::store(y + ((size_t)(t0 + tt) * n_heads + h) * n + col, v);
+  }
 }
 
 template <typename TX, typename TW, typename TY>
 static void launch_heads_linear(const void* x, const void* w, void* y, int n_tokens, int n_heads, int n, int k, hipStream_t s) {
   dim3 grid((n_tokens + HL_TOKENS - 1) / HL_TOKENS, n_heads, (n + RB_WAVE - 1) / RB_WAVE);
-  heads_linear_kernel<TX, TW, TY><<<grid, RB_WAVE, (size_t)HL_TOKENS * k * sizeof(float), s>>>((const TX*)x, (const TW*)w, (TY*)y,
-                                                                                               n_tokens, n_heads, n, k);
+  const size_t lds = ((size_t)HL_TOKENS * k + (size_t)(HL_WAVES - 1) * HL_TOKENS * RB_WAVE) * sizeof(float);
+  heads_linear_kernel<TX, TW, TY><<<grid, RB_WAVE * HL_WAVES, lds, s>>>((const TX*)x, (const TW*)w, (TY*)y, n_tokens, n_heads, n, k);
 }
 
 extern "C" int rb_heads_linear(const void* x, int x_dtype, const void* w, int w_dtype, void* y, int y_dtype, int n_tokens,
                                int n_heads, int n, int k, void* stream) {
   RB_RECORDED(rb_heads_linear(x, x_dtype, w, w_dtype, y, y_dtype, n_tokens, n_heads, n, k, stream));
   RB_REQUIRE(n_tokens >= 0 && n_heads > 0 && n_heads <= 65535 && n > 0 && n <= 65535 * 64 && k > 0, "rb_heads_linear: bad sizes");
-  RB_REQUIRE(k <= 1024, "rb_heads_linear: inner size %d not supported (at most 1024)", k);
+  RB_REQUIRE(k <= 768, "rb_heads_linear: inner size %d not supported (at most 768)", k);
   if (n_tokens == 0) return 0;
   hipStream_t s = (hipStream_t)stream;
   const int key = x_dtype * 4 + w_dtype * 2 + y_dtype;

@@ -152,6 +152,7 @@ class Kernels:
             "rb_attention_decode_bf16_sinks": [_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _F, _I, _I, _P, _P, _P],
             "rb_embed_streams": [_P, _I, _P, _P, _I, _L, _I, _I, _P],
             "rb_streams_layernorm": [_P, _I, _L, _P, _P, _P, _P, _F, _P, _I, _I, _P, _I, _P],
+            "rb_streams_update_layernorm": [_P, _I, _L, _P, _P, _P, _P, _P, _P, _P, _P, _F, _P, _I, _I, _P, _I, _P],
             "rb_streams_update": [_P, _I, _L, _P, _P, _P, _P, _I, _I, _P],
             "rb_xielu": [_P, _P, _P, _I, _L, _P],
             "rb_tanh_cap": [_P, _F, _L, _P],
@@ -447,8 +448,10 @@ class Kernels:
 
     def streams_layernorm(self, x: torch.Tensor, coef: Optional[torch.Tensor], weight: torch.Tensor,
                           bias: Optional[torch.Tensor], eps: float, rows: Optional[torch.Tensor], out: torch.Tensor,
-                          delta: Optional[torch.Tensor] = None) -> None:
-        """x [S, T, E] (or [T, E]: one stream) float32; out [rows or T, E]: the layer norm of sum_s coef[s] x[s]."""
+                          delta: Optional[torch.Tensor] = None, update=None) -> None:
+        """x [S, T, E] (or [T, E]: one stream) float32; out [rows or T, E]: the layer norm of sum_s coef[s] x[s].
+        update (mix [S, S], out_coef [S], y [T, E], scale [E] or None): `streams_update` with these first, in the same
+        pass (every row, so rows must be None)."""
         if x.dim() == 2:
             x = x.unsqueeze(0)
         s_, n, width = x.shape
@@ -465,9 +468,19 @@ class Kernels:
             n_rows = rows.shape[0]
             _check(rows, "rows", torch.int32, (n_rows,))
         _check(out, "out", None, (n_rows, width))
-        self._ok(self._lib.rb_streams_layernorm(_ptr(x), s_, n * width, _ptr(coef), _ptr(delta), _ptr(weight), _ptr(bias),
-                                                float(eps), _ptr(rows), n_rows, width, _ptr(out), dtype_code(out.dtype),
-                                                self._stream()))
+        mix = out_coef = y = scale = None
+        if update is not None:
+            mix, out_coef, y, scale = update
+            if rows is not None:
+                raise KernelError("streams_layernorm: an update takes every row")
+            _check(mix, "mix", torch.float32, (s_, s_))
+            _check(out_coef, "out_coef", torch.float32, (s_,))
+            _check(y, "y", torch.float32, (n, width))
+            if scale is not None:
+                _check(scale, "scale", torch.float32, (width,))
+        self._ok(self._lib.rb_streams_update_layernorm(_ptr(x), s_, n * width, _ptr(mix), _ptr(out_coef), _ptr(y), _ptr(scale),
+                                                       _ptr(coef), _ptr(delta), _ptr(weight), _ptr(bias), float(eps), _ptr(rows),
+                                                       n_rows, width, _ptr(out), dtype_code(out.dtype), self._stream()))
 
     def streams_update(self, x: torch.Tensor, mix: torch.Tensor, out_coef: torch.Tensor, y: torch.Tensor,
                        scale: Optional[torch.Tensor]) -> None:

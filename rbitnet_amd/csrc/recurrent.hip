@@ -143,11 +143,23 @@ extern "C" int rb_delta_prep(float* qk, long long qk_stride, int n_kv_heads, int
 // Per sequence and head, token after token:
 //   S <- diag(g) S;  u = beta (v - S^T k);  S <- S + k u^T;  o = S^T q
 // The columns of S (one per value channel) do not meet: a column is held by RG lanes, each with DKL of its rows in
-// registers; the two dot products over the rows are finished by shuffles among the RG lanes.  A workgroup is one wave
+// registers; the dot products over the rows are finished among the RG lanes by moves inside a row of lanes.  A workgroup is one wave
 // and holds 64 / RG columns.  Tokens go by in chunks of CH: q, k, g, v and beta of a chunk lie in LDS for all lanes, and
 // the next chunk's loads are in flight (in registers) while the current one is computed, so that a token costs its
 // arithmetic and no trip to memory; the chunk's outputs leave through LDS as whole rows.  The state is read once and
 // written once.
+// The sum over each group of RG neighbouring lanes (RG = 4, 8 or 16), in every lane of the group, by moves inside a
+// row of 16 lanes (no trip through LDS): the two swaps inside a quad, then the mirror of a half row, then of a row.
+template <int RG>
+__device__ __forceinline__ float lanes_sum(float v) {
+  static_assert(RG == 4 || RG == 8 || RG == 16, "groups of 4, 8 or 16 lanes");
+  v += __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), 0xB1, 0xF, 0xF, true));   // quad_perm [1,0,3,2]
+  v += __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), 0x4E, 0xF, 0xF, true));   // quad_perm [2,3,0,1]
+  if (RG >= 8) v += __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), 0x141, 0xF, 0xF, true));   // row_half_mirror
+  if (RG >= 16) v += __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), 0x140, 0xF, 0xF, true));  // row_mirror
+  return v;
+}
+
 template <int DKL, int RG, int CH>
 __global__ __launch_bounds__(RB_WAVE) void delta_rule_kernel(
     const float* __restrict__ q, const float* __restrict__ k, size_t qk_stride, const float* __restrict__ v,
@@ -212,27 +224,40 @@ __global__ __launch_bounds__(RB_WAVE) void delta_rule_kernel(
     if (lane < CH) sb[lane] = rb;
     __syncthreads();
     if (t0 + CH < n) fetch(t0 + CH);                   // in flight while this chunk is computed
-    for (int tt = 0; tt < nt; ++tt) {
+    // One token: with D = diag(g) S and u = beta (v - D^T k), the read-out of the updated state is
+    // (D + k u^T)^T q = D^T q + u (k . q): one pass over the decayed column gives both dot products, and a token has
+    // one reduction among the RG lanes on its way instead of two.  Two partial sums each: shorter chains of additions.
+    auto token = [&](int tt) {
       const float vv = sv[tt][lane / RG];
       const float bt = sb[tt];
-      float kv = 0.f;
+      float kv0 = 0.f, kv1 = 0.f, dq0 = 0.f, dq1 = 0.f, kq0 = 0.f, kq1 = 0.f;
 #pragma unroll
-      for (int i = 0; i < DKL; ++i) {
+      for (int i = 0; i < DKL; i += 2) {
+        const float k0 = sk[tt][rg * DKL + i], q0 = sq[tt][rg * DKL + i];
+        const float k1 = sk[tt][rg * DKL + i + 1], q1 = sq[tt][rg * DKL + i + 1];
         s[i] *= sg[tt][rg * DKL + i];
-        kv = fmaf(s[i], sk[tt][rg * DKL + i], kv);
+        s[i + 1] *= sg[tt][rg * DKL + i + 1];
+        kv0 = fmaf(s[i], k0, kv0);
+        kv1 = fmaf(s[i + 1], k1, kv1);
+        dq0 = fmaf(s[i], q0, dq0);
+        dq1 = fmaf(s[i + 1], q1, dq1);
+        kq0 = fmaf(k0, q0, kq0);
+        kq1 = fmaf(k1, q1, kq1);
       }
-#pragma unroll
-      for (int o = 1; o < RG; o <<= 1) kv += __shfl_xor(kv, o, RB_WAVE);
+      const float kv = lanes_sum<RG>(kv0 + kv1);
+      const float dq = lanes_sum<RG>(dq0 + dq1);
+      const float kq = lanes_sum<RG>(kq0 + kq1);
       const float u = bt * (vv - kv);
-      float oq = 0.f;
 #pragma unroll
-      for (int i = 0; i < DKL; ++i) {
-        s[i] = fmaf(sk[tt][rg * DKL + i], u, s[i]);
-        oq = fmaf(s[i], sq[tt][rg * DKL + i], oq);
-      }
+      for (int i = 0; i < DKL; ++i) s[i] = fmaf(sk[tt][rg * DKL + i], u, s[i]);
+      if (rg == 0) so[tt][lane / RG] = fmaf(u, kq, dq);
+    };
+    if (nt == CH) {
+      // a whole chunk as straight code, so that a token's reads from LDS are issued while the one before is computed
 #pragma unroll
-      for (int o = 1; o < RG; o <<= 1) oq += __shfl_xor(oq, o, RB_WAVE);
-      if (rg == 0) so[tt][lane / RG] = oq;
+      for (int tt = 0; tt < CH; ++tt) token(tt);
+    } else {
+      for (int tt = 0; tt < nt; ++tt) token(tt);
     }
     __syncthreads();
     for (int e = lane; e < nt * COLS; e += RB_WAVE) {
@@ -253,7 +278,7 @@ static void launch_delta_rule(const float* q, const float* k, size_t qk_stride, 
                               const int32_t* slots, float* out, int n_seqs, int n_heads, int n_kv, int dim, int vdim,
                               hipStream_t s) {
   constexpr int COLS = RB_WAVE / RG;
-  static_assert((DKL * RG * CH) % RB_WAVE == 0 && CH <= RB_WAVE, "a chunk's values are dealt evenly to the lanes");
+  static_assert((DKL * RG * CH) % RB_WAVE == 0 && CH <= RB_WAVE && DKL % 2 == 0, "a chunk's values are dealt evenly to the lanes");
   dim3 grid(n_seqs, n_heads, (vdim + COLS - 1) / COLS);
   delta_rule_kernel<DKL, RG, CH><<<grid, RB_WAVE, 0, s>>>(q, k, qk_stride, v, v_stride, g, g_stride, beta, state, cu_seqlens,
                                                           slots, out, n_heads, n_kv, dim, vdim);
@@ -275,17 +300,23 @@ extern "C" int rb_delta_rule(const float* q, const float* k, long long qk_stride
   const size_t qs = (size_t)qk_stride, vs = (size_t)v_stride;
 #define DR_GO(DKL, RG, CH) \
   launch_delta_rule<DKL, RG, CH>(q, k, qs, v, vs, g, (size_t)g_stride, beta, state, cu_seqlens, slots, out, n_seqs, n_heads, n_kv_heads, dim, vdim, s)
-  // rows of a column over RG lanes: short chains per token, and enough waves for the GPU while sequences are few;
-  // chunks as long as the registers that hold the next one allow
+  // Rows of a column over RG lanes, chunks as long as the registers that hold the next one allow.  A token's time is
+  // its lane's share of the column, so while the waves do not fill the GPU's SIMDs a column goes to more lanes
+  // (more and shorter waves); once they do, fewer lanes per column save the moves between them.
+  const long long simds = 4LL * rb_compute_units();
+  auto waves = [&](int rg) { return (long long)n_seqs * n_heads * ((vdim + RB_WAVE / rg - 1) / (RB_WAVE / rg)); };
   if (dim <= 16)
     DR_GO(4, 4, 16);
-  else if (dim <= 32)
-    DR_GO(8, 4, 16);
-  else if (dim <= 64)
-    DR_GO(8, 8, 16);
-  else if (dim <= 128)
-    DR_GO(16, 8, 16);
-  else if (dim <= 256)
+  else if (dim <= 32) {
+    if (waves(4) >= simds) DR_GO(8, 4, 16);
+    else DR_GO(4, 8, 16);
+  } else if (dim <= 64) {
+    if (waves(8) >= simds) DR_GO(8, 8, 16);
+    else DR_GO(4, 16, 16);
+  } else if (dim <= 128) {
+    if (waves(8) >= simds) DR_GO(16, 8, 16);
+    else DR_GO(8, 16, 16);
+  } else if (dim <= 256)
     DR_GO(16, 16, 8);
   else
     DR_GO(32, 16, 4);

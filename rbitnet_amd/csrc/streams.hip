@@ -20,7 +20,9 @@ template <typename TO>
 __global__ void streams_layernorm_kernel(float* __restrict__ x, int n_streams, size_t stream_stride,
                                          const float* __restrict__ coef, const float* __restrict__ delta,
                                          const float* __restrict__ weight, const float* __restrict__ bias, float eps,
-                                         const int32_t* __restrict__ rows, int width, TO* __restrict__ out) {
+                                         const int32_t* __restrict__ rows, int width, TO* __restrict__ out,
+                                         const float* __restrict__ mix, const float* __restrict__ out_coef,
+                                         const float* __restrict__ y, const float* __restrict__ scale) {
   extern __shared__ float u[];
   __shared__ float scratch[16];
   const int r = blockIdx.x;
@@ -29,9 +31,30 @@ __global__ void streams_layernorm_kernel(float* __restrict__ x, int n_streams, s
   float sum = 0.f;
   for (int j = threadIdx.x; j < width; j += blockDim.x) {
     float v = 0.f;
-    for (int s = 0; s < n_streams; ++s) {
-      const float xv = x[(size_t)s * stream_stride + src * width + j];
-      v = coef ? fmaf(coef[s], xv, v) : v + xv;
+    if (mix) {
+      // the update that was still to be done: every copy from all the old ones, then the mixture of the new ones
+      float old[ST_MAX_STREAMS];
+#pragma unroll
+      for (int s = 0; s < ST_MAX_STREAMS; ++s)
+        if (s < n_streams) old[s] = x[(size_t)s * stream_stride + src * width + j];
+      float yv = y[src * width + j];
+      if (scale) yv *= scale[j];
+#pragma unroll
+      for (int k = 0; k < ST_MAX_STREAMS; ++k) {
+        if (k < n_streams) {
+          float nv = out_coef[k] * yv;
+#pragma unroll
+          for (int s = 0; s < ST_MAX_STREAMS; ++s)
+            if (s < n_streams) nv = fmaf(mix[s * n_streams + k], old[s], nv);
+          x[(size_t)k * stream_stride + src * width + j] = nv;
+          v = coef ? fmaf(coef[k], nv, v) : v + nv;
+        }
+      }
+    } else {
+      for (int s = 0; s < n_streams; ++s) {
+        const float xv = x[(size_t)s * stream_stride + src * width + j];
+        v = coef ? fmaf(coef[s], xv, v) : v + xv;
+      }
     }
     if (delta) v += delta[src * width + j];
     if (write_back) x[src * width + j] = v;
@@ -52,23 +75,140 @@ __global__ void streams_layernorm_kernel(float* __restrict__ x, int n_streams, s
   }
 }
 
+// The same for widths that are multiples of 4, four values a thread with 16-byte loads and up to 1024 threads a row,
+// so that a row's loads are all in flight together (a step of few tokens has few rows, and their time is the
+// chain of trips to memory).
+__device__ __forceinline__ float4 ld4(const float* p) { return *reinterpret_cast<const float4*>(p); }
+__device__ __forceinline__ float4 fma4(float a, const float4& b, const float4& c) {
+  return make_float4(fmaf(a, b.x, c.x), fmaf(a, b.y, c.y), fmaf(a, b.z, c.z), fmaf(a, b.w, c.w));
+}
+__device__ __forceinline__ void st4(float* p, float a, float b, float c, float d) { *reinterpret_cast<float4*>(p) = make_float4(a, b, c, d); }
+__device__ __forceinline__ void st4(bf16_t* p, float a, float b, float c, float d) {
+  *reinterpret_cast<uint2*>(p) = make_uint2(pack_bf16x2(a, b), pack_bf16x2(c, d));
+}
+
+template <typename TO>
+__global__ __launch_bounds__(1024) void streams_layernorm_vec_kernel(
+    float* __restrict__ x, int n_streams, size_t stream_stride, const float* __restrict__ coef, const float* __restrict__ delta,
+    const float* __restrict__ weight, const float* __restrict__ bias, float eps, const int32_t* __restrict__ rows, int width,
+    TO* __restrict__ out, const float* __restrict__ mix, const float* __restrict__ out_coef, const float* __restrict__ y,
+    const float* __restrict__ scale) {
+  extern __shared__ float u[];
+  __shared__ float scratch[16];
+  __shared__ float c_mix[ST_MAX_STREAMS * ST_MAX_STREAMS], c_out[ST_MAX_STREAMS], c_in[ST_MAX_STREAMS];
+  const int r = blockIdx.x;
+  const size_t src = rows ? (size_t)rows[r] : (size_t)r;
+  const bool write_back = delta != nullptr && rows == nullptr && n_streams == 1;
+  if ((int)threadIdx.x < n_streams) {
+    c_in[threadIdx.x] = coef ? coef[threadIdx.x] : 1.0f;
+    if (mix) c_out[threadIdx.x] = out_coef[threadIdx.x];
+  }
+  if (mix && (int)threadIdx.x < n_streams * n_streams) c_mix[threadIdx.x] = mix[threadIdx.x];
+  __syncthreads();
+  float sum = 0.f;
+  for (int j = 4 * threadIdx.x; j < width; j += 4 * blockDim.x) {
+    float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (mix) {
+      float4 old[ST_MAX_STREAMS];
+#pragma unroll
+      for (int s = 0; s < ST_MAX_STREAMS; ++s)
+        if (s < n_streams) old[s] = ld4(x + (size_t)s * stream_stride + src * width + j);
+      float4 yv = ld4(y + src * width + j);
+      if (scale) {
+        const float4 sc = ld4(scale + j);
+        yv = make_float4(yv.x * sc.x, yv.y * sc.y, yv.z * sc.z, yv.w * sc.w);
+      }
+#pragma unroll
+      for (int k = 0; k < ST_MAX_STREAMS; ++k) {
+        if (k < n_streams) {
+          const float oc = c_out[k];
+          float4 nv = make_float4(oc * yv.x, oc * yv.y, oc * yv.z, oc * yv.w);
+#pragma unroll
+          for (int s = 0; s < ST_MAX_STREAMS; ++s)
+            if (s < n_streams) nv = fma4(c_mix[s * n_streams + k], old[s], nv);
+          *reinterpret_cast<float4*>(x + (size_t)k * stream_stride + src * width + j) = nv;
+          v = fma4(c_in[k], nv, v);
+        }
+      }
+    } else {
+#pragma unroll
+      for (int s = 0; s < ST_MAX_STREAMS; ++s)
+        if (s < n_streams) v = fma4(c_in[s], ld4(x + (size_t)s * stream_stride + src * width + j), v);
+    }
+    if (delta) {
+      const float4 d = ld4(delta + src * width + j);
+      v = make_float4(v.x + d.x, v.y + d.y, v.z + d.z, v.w + d.w);
+    }
+    if (write_back) *reinterpret_cast<float4*>(x + src * width + j) = v;
+    *reinterpret_cast<float4*>(u + j) = v;
+    sum += (v.x + v.y) + (v.z + v.w);
+  }
+  const float mean = block_sum(sum, scratch) / (float)width;
+  float ss = 0.f;
+  for (int j = 4 * threadIdx.x; j < width; j += 4 * blockDim.x) {
+    const float4 v = *reinterpret_cast<const float4*>(u + j);
+    const float a = v.x - mean, b = v.y - mean, c = v.z - mean, d = v.w - mean;
+    ss += (a * a + b * b) + (c * c + d * d);
+  }
+  const float f = 1.0f / sqrtf(block_sum(ss, scratch) / (float)width + eps);
+  TO* orow = out + (size_t)r * width;
+  for (int j = 4 * threadIdx.x; j < width; j += 4 * blockDim.x) {
+    const float4 v = *reinterpret_cast<const float4*>(u + j);
+    const float4 wv = ld4(weight + j);
+    float4 o = make_float4((v.x - mean) * f * wv.x, (v.y - mean) * f * wv.y, (v.z - mean) * f * wv.z, (v.w - mean) * f * wv.w);
+    if (bias) {
+      const float4 bv = ld4(bias + j);
+      o = make_float4(o.x + bv.x, o.y + bv.y, o.z + bv.z, o.w + bv.w);
+    }
+    st4(orow + j, o.x, o.y, o.z, o.w);
+  }
+}
+
 extern "C" int rb_streams_layernorm(float* x, int n_streams, long long stream_stride, const float* coef,
                                     const float* delta, const float* weight, const float* bias, float eps,
                                     const int32_t* rows, int n_rows, int width, void* out, int out_dtype, void* stream) {
-  RB_RECORDED(rb_streams_layernorm(x, n_streams, stream_stride, coef, delta, weight, bias, eps, rows, n_rows, width, out,
-                                   out_dtype, stream));
+  return rb_streams_update_layernorm(x, n_streams, stream_stride, nullptr, nullptr, nullptr, nullptr, coef, delta, weight, bias,
+                                     eps, rows, n_rows, width, out, out_dtype, stream);
+}
+
+// The same after an update of the copies that was still to be done (rb_streams_update's mix, out_coef, y, scale; mix
+// null: none), in one pass over the rows: the copies are rewritten and the norm reads the new ones.  With an update
+// every row is taken (rows must be null).
+extern "C" int rb_streams_update_layernorm(float* x, int n_streams, long long stream_stride, const float* mix,
+                                           const float* out_coef, const float* y, const float* scale, const float* coef,
+                                           const float* delta, const float* weight, const float* bias, float eps,
+                                           const int32_t* rows, int n_rows, int width, void* out, int out_dtype,
+                                           void* stream) {
+  RB_RECORDED(rb_streams_update_layernorm(x, n_streams, stream_stride, mix, out_coef, y, scale, coef, delta, weight, bias, eps,
+                                          rows, n_rows, width, out, out_dtype, stream));
+  RB_REQUIRE(mix == nullptr || (rows == nullptr && out_coef != nullptr && y != nullptr),
+             "rb_streams_update_layernorm: an update takes every row and needs out_coef and y");
   RB_REQUIRE(n_rows >= 0 && width > 0 && width <= 16384, "rb_streams_layernorm: bad sizes %d x %d (width at most 16384)", n_rows, width);
   RB_REQUIRE(n_streams >= 1 && n_streams <= ST_MAX_STREAMS && stream_stride >= 0, "rb_streams_layernorm: %d streams (1 to %d)",
              n_streams, ST_MAX_STREAMS);
   if (n_rows == 0) return 0;
   hipStream_t s = (hipStream_t)stream;
   const size_t lds = (size_t)width * sizeof(float);
+  auto aligned = [](const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; };
+  if (width % 4 == 0 && stream_stride % 4 == 0 && aligned(x) && aligned(delta) && aligned(weight) && aligned(bias) && aligned(out) &&
+      aligned(y) && aligned(scale) && (out_dtype == RB_F32 || out_dtype == RB_BF16)) {
+    int threads = ((width / 4 + RB_WAVE - 1) / RB_WAVE) * RB_WAVE;
+    if (threads > 1024) threads = 1024;
+    if (out_dtype == RB_F32)
+      streams_layernorm_vec_kernel<float><<<n_rows, threads, lds, s>>>(x, n_streams, (size_t)stream_stride, coef, delta, weight, bias,
+                                                                       eps, rows, width, (float*)out, mix, out_coef, y, scale);
+    else
+      streams_layernorm_vec_kernel<bf16_t><<<n_rows, threads, lds, s>>>(x, n_streams, (size_t)stream_stride, coef, delta, weight,
+                                                                        bias, eps, rows, width, (bf16_t*)out, mix, out_coef, y, scale);
+    RB_LAUNCH_CHECK();
+    return 0;
+  }
   if (out_dtype == RB_F32)
     streams_layernorm_kernel<float><<<n_rows, 256, lds, s>>>(x, n_streams, (size_t)stream_stride, coef, delta, weight, bias, eps,
-                                                             rows, width, (float*)out);
+                                                             rows, width, (float*)out, mix, out_coef, y, scale);
   else if (out_dtype == RB_BF16)
     streams_layernorm_kernel<bf16_t><<<n_rows, 256, lds, s>>>(x, n_streams, (size_t)stream_stride, coef, delta, weight, bias, eps,
-                                                              rows, width, (bf16_t*)out);
+                                                              rows, width, (bf16_t*)out, mix, out_coef, y, scale);
   else
     RB_REQUIRE(false, "rb_streams_layernorm: unknown dtype %d", out_dtype);
   RB_LAUNCH_CHECK();
@@ -146,23 +286,37 @@ extern "C" int rb_embed_streams(const void* table, int table_dtype, const int32_
 
 // ---------------------------------------------------------------- xIELU
 // z > 0: softplus(p) z^2 + z / 2;  z <= 0: (1/2 + softplus(q)) (exp(z) - 1 - z) + z / 2, with (p, q) = act[0..1].
+__device__ __forceinline__ float xielu_value(float v, float ap, float an) {
+  return v > 0.f ? fmaf(ap * v, v, 0.5f * v) : fmaf(an, expm1f(v) - v, 0.5f * v);
+}
+__device__ __forceinline__ void xielu_store4(float* p, float a, float b, float c, float d) {
+  *reinterpret_cast<float4*>(p) = make_float4(a, b, c, d);
+}
+__device__ __forceinline__ void xielu_store4(bf16_t* p, float a, float b, float c, float d) {
+  *reinterpret_cast<uint2*>(p) = make_uint2(pack_bf16x2(a, b), pack_bf16x2(c, d));
+}
+
+// four values a thread with 16-byte loads (n4 quads), then the rest one by one
 template <typename TO>
 __global__ void xielu_kernel(const float* __restrict__ z, const float* __restrict__ act, TO* __restrict__ out, size_t n) {
   const float p = act[0], q = act[1];
   const float ap = p > 20.0f ? p : log1pf(expf(p));
   const float an = 0.5f + (q > 20.0f ? q : log1pf(expf(q)));
-  for (size_t e = (size_t)blockIdx.x * blockDim.x + threadIdx.x; e < n; e += (size_t)gridDim.x * blockDim.x) {
-    const float v = z[e];
-    const float r = v > 0.f ? fmaf(ap * v, v, 0.5f * v) : fmaf(an, expm1f(v) - v, 0.5f * v);
-    Num<TO>::store(out + e, r);
+  const size_t n4 = n / 4;
+  for (size_t e = (size_t)blockIdx.x * blockDim.x + threadIdx.x; e < n4; e += (size_t)gridDim.x * blockDim.x) {
+    const float4 v = *reinterpret_cast<const float4*>(z + 4 * e);
+    xielu_store4(out + 4 * e, xielu_value(v.x, ap, an), xielu_value(v.y, ap, an), xielu_value(v.z, ap, an),
+                 xielu_value(v.w, ap, an));
   }
+  for (size_t e = 4 * n4 + (size_t)blockIdx.x * blockDim.x + threadIdx.x; e < n; e += (size_t)gridDim.x * blockDim.x)
+    Num<TO>::store(out + e, xielu_value(z[e], ap, an));
 }
 
 extern "C" int rb_xielu(const float* z, const float* act, void* out, int out_dtype, long long n, void* stream) {
   RB_RECORDED(rb_xielu(z, act, out, out_dtype, n, stream));
   RB_REQUIRE(n >= 0, "rb_xielu: bad size");
   if (n == 0) return 0;
-  const size_t blocks = ((size_t)n + 255) / 256;
+  const size_t blocks = ((size_t)n / 4 + 255) / 256 + 1;
   const int grid = (int)(blocks < 65535 ? blocks : 65535);
   hipStream_t s = (hipStream_t)stream;
   if (out_dtype == RB_F32)

@@ -6,6 +6,8 @@ The stream is x [S, T, E] float32, all copies equal to the embedding at the star
 (from, to) and ls<p> [E]:
     u = sum_s in[s] x_s;   h = norm<p>(u);   (p = 1, with a convolution: h <- h + conv(h), causal, per channel)
     y = ls<p> * sublayer(h);   x_j <- sum_s mix[s, j] x_s + out[j] * y   for all j at once
+The update of the copies is left to the norm that reads the stream next (`StreamsUpdate`: the layer's own second
+norm, the next layer's first, the head's), which does it in its own pass over the rows.
 What reads the stream after the last layer takes the sum of the copies (the head's norm does).  One copy with
 in = out = mix = 1 is the plain pre-norm layer.  Norms, mixtures and sums in float32.
 
@@ -24,6 +26,7 @@ import torch
 from ..errors import ConfigError
 from .base import BuildEnv, CacheRequest, Part, TensorSpec, build_part, register_block
 from .short_conv import ACT_NONE, ShortConv
+from .stream import StreamsUpdate
 
 DEFAULT_SEGMENTS = {"norm1": "norm1", "mixer": "mix", "norm2": "norm2", "feed_forward": "mlp"}
 DEFAULT_NAMES = {"in": "hc{p}.in", "out": "hc{p}.out", "mix": "hc{p}.mix", "scale": "ls{p}"}
@@ -112,29 +115,32 @@ class HyperBlock:
                 out.append(req)
         return out
 
-    def _norm(self, norm, x: torch.Tensor, coef: torch.Tensor, out_dtype) -> torch.Tensor:
+    def _norm(self, norm, x: torch.Tensor, pending, coef: torch.Tensor, out_dtype) -> torch.Tensor:
+        """norm(sum_s coef[s] x_s), after the update that the sublayer before left to be done (in the same pass)."""
         if x.dim() == 3 and hasattr(norm, "names"):           # a norm that reads the mixture of the copies itself
-            return norm.forward(x, None, None, coef=coef, out_dtype=out_dtype)
+            return norm.forward(x, pending, None, coef=coef, out_dtype=out_dtype)
         raise ConfigError("this arrangement needs a norm that reads a stream in several copies (layernorm)")
 
     def forward(self, x: torch.Tensor, pending, ctx, view, next_norm=None):
         if x.dim() != 3 or x.shape[0] != self.streams:
             raise ConfigError(f"the stream must come in {self.streams} copies [S, T, E] (the embedding's `streams`)")
+        if pending is not None and not isinstance(pending, StreamsUpdate):
+            raise ConfigError("a layer with the stream in several copies cannot follow one that leaves a plain term to be added")
         lib, dt = self.env.lib, self.env.dtype
         c = self.coef[1]
         if self.conv is not None:
-            hn = self._norm(self.norm1, x, c["in"], torch.float32)
+            hn = self._norm(self.norm1, x, pending, c["in"], torch.float32)
             h = self.conv.forward(hn, ctx, view.states.get("input_conv"), dt)
         else:
-            h = self._norm(self.norm1, x, c["in"], dt)
+            h = self._norm(self.norm1, x, pending, c["in"], dt)
         y = self.mixer.forward(h, ctx, view)
-        lib.streams_update(x, c["mix"], c["out"], y, c["scale"])
+        pending = StreamsUpdate(lib, c["mix"], c["out"], y, c["scale"])
         if self.feed_forward is not None:
             c = self.coef[2]
-            h = self._norm(self.norm2, x, c["in"], dt)
+            h = self._norm(self.norm2, x, pending, c["in"], dt)
             y = self.feed_forward.forward(h, ctx)
-            lib.streams_update(x, c["mix"], c["out"], y, c["scale"])
-        return None
+            pending = StreamsUpdate(lib, c["mix"], c["out"], y, c["scale"])
+        return pending                                        # done by whichever norm reads the stream next
 
 
 register_block("hyper", HyperBlock)

@@ -49,6 +49,8 @@ class LatentAttention(Part):
             raise ConfigError(f"latent attention: kv_rank {self.kv_rank} not supported (even, at most {MAX_RANK})")
         if min(self.heads, self.dim, self.vdim, self.q_rank) <= 0:
             raise ConfigError("latent attention: sizes must be positive")
+        if self.dim > 768:
+            raise ConfigError(f"latent attention: head size {self.dim} not supported (at most 768)")
         self.names = dict(DEFAULT_NAMES, **(params.get("names") or {}))
         self.hidden = env.hidden_size
 

@@ -24,7 +24,7 @@ from typing import Dict, Optional
 import torch
 
 from .base import BuildEnv, Part, TensorSpec, register_norm
-from .stream import GainedRows  # noqa: F401  (its old home; importers find it here too)
+from .stream import GainedRows, StreamsUpdate  # noqa: F401  (GainedRows: its old home; importers find it here too)
 
 
 class RMSNorm(Part):
@@ -89,7 +89,14 @@ class LayerNorm(Part):
         t = x.shape[-2]
         n = t if rows is None else rows.shape[0]
         out = torch.empty((n, self.size), dtype=out_dtype or self.env.dtype, device=x.device)
-        self.env.lib.streams_layernorm(x, coef, self.weight, self.bias, self.eps, rows, out, delta=delta)
+        update = None
+        if isinstance(delta, StreamsUpdate):              # an update of the copies still to be done
+            if rows is None:
+                update, delta = delta.parts(), None       # in this norm's own pass over the rows
+            else:
+                delta.apply(x)                            # only some rows are normalised: all are updated first
+                delta = None
+        self.env.lib.streams_layernorm(x, coef, self.weight, self.bias, self.eps, rows, out, delta=delta, update=update)
         return out
 
 

@@ -12,6 +12,8 @@ prepared for the norm that follows, `GainedRows`).  What a sublayer has not yet 
     tensor [T, E]   a float32 term still to be added
     tensor [P,T,E]  P terms, the K slices of a product, to be added up in their order
     GainedRows      nothing to add, and the rows as the next norm's kernel would read them
+    StreamsUpdate   (a stream kept in several copies [S, T, E]) the update of all copies by a sublayer's result that
+                    is still to be done; a norm that reads such a stream does it in its own pass over the rows
 
 What a part or a norm can do, it says with class attributes; a part without any gets and
 returns plain tensors, a norm without any does every sum and every normalisation in its own
@@ -64,6 +66,21 @@ class GainedRows:
 
     def tensor(self) -> torch.Tensor:
         return self.norm.forward(self.x, None, self.rows)
+
+
+class StreamsUpdate:
+    """What a sublayer left to be done to a stream in several copies x [S, T, E]:
+    x_j <- sum_s mix[s, j] x_s + out_coef[j] * (scale * y) for all j at once.  apply() does it with the kernel of its
+    own; a norm that reads such streams (`layernorm`) takes it as `delta` and does it while it normalises."""
+
+    def __init__(self, lib, mix: torch.Tensor, out_coef: torch.Tensor, y: torch.Tensor, scale: Optional[torch.Tensor]):
+        self.lib, self.mix, self.out_coef, self.y, self.scale = lib, mix, out_coef, y, scale
+
+    def parts(self):
+        return self.mix, self.out_coef, self.y, self.scale
+
+    def apply(self, x: torch.Tensor) -> None:
+        self.lib.streams_update(x, self.mix, self.out_coef, self.y, self.scale)
 
 
 def normed_for(part, norm, x: torch.Tensor, pending, rows: Optional[torch.Tensor] = None):
