@@ -66,7 +66,8 @@ extern "C" int rb_latent_norm_store(const float* proj, long long stride, int q_r
 // y[t, h, n] = sum_k w[h, k, n] * x[t, h, k]: H small matrices, stored [H, K, N] (the output index runs fastest, so
 // that neighbouring lanes read neighbouring weights).  A workgroup of four waves takes HL_TOKENS tokens and 64 output
 // columns of one head: the tokens' inputs in LDS, a lane per column with one sum per token; the waves share the inner
-// index (wave w takes k = w, w + 4, ...), sixteen weights in flight per lane, and add up through LDS in a fixed order.
+// index (wave w takes k = w, w + 4, ...), sixteen weights in flight per lane (the scheduler is told not to move a load
+// down to its use: it would trade the registers for a trip to memory per weight), and add up through LDS in a fixed order.
 #define HL_TOKENS 16
 #define HL_WAVES 4
 template <typename TX, typename TW, typename TY>
@@ -77,9 +78,21 @@ __global__ __launch_bounds__(RB_WAVE * HL_WAVES) void heads_linear_kernel(const 
   const int t0 = blockIdx.x * HL_TOKENS, h = blockIdx.y;
   const int lane = threadIdx.x & (RB_WAVE - 1), wave = threadIdx.x / RB_WAVE;
   const int nt = n_tokens - t0 < HL_TOKENS ? n_tokens - t0 : HL_TOKENS;
-  for (int idx = threadIdx.x; idx < HL_TOKENS * k; idx += RB_WAVE * HL_WAVES) {
-    const int tt = idx / k, kk = idx - tt * k;
-    xs[idx] = tt < nt ? Num<TX>::load(x + ((size_t)(t0 + tt) * n_heads + h) * k + kk) : 0.f;
+  // the tokens' inputs, eight loads in flight per lane (a step of few tokens is a chain of trips to memory otherwise)
+  for (int base = 0; base < HL_TOKENS * k; base += 8 * RB_WAVE * HL_WAVES) {
+    float v[8];
+#pragma unroll
+    for (int it = 0; it < 8; ++it) {
+      const int idx = base + it * RB_WAVE * HL_WAVES + threadIdx.x;
+      const int tt = idx / k, kk = idx - tt * k;
+      v[it] = (idx < HL_TOKENS * k && tt < nt) ? Num<TX>::load(x + ((size_t)(t0 + tt) * n_heads + h) * k + kk) : 0.f;
+    }
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int it = 0; it < 8; ++it) {
+      const int idx = base + it * RB_WAVE * HL_WAVES + threadIdx.x;
+      if (idx < HL_TOKENS * k) xs[idx] = v[it];
+    }
   }
   __syncthreads();
   const int col = blockIdx.z * RB_WAVE + lane;
@@ -93,6 +106,7 @@ __global__ __launch_bounds__(RB_WAVE * HL_WAVES) void heads_linear_kernel(const 
     float wv[16];
 #pragma unroll
     for (int j = 0; j < 16; ++j) wv[j] = Num<TW>::load(wh + (size_t)(kk + j * HL_WAVES) * n);
+    __builtin_amdgcn_sched_barrier(0);          // all sixteen loads are issued before the first is waited for
 #pragma unroll
     for (int j = 0; j < 16; ++j)
 #pragma unroll

@@ -100,7 +100,7 @@ extern "C" int rb_short_conv(const float* x, long long x_stride, const float* w,
 // ---------------------------------------------------------------- gated delta rule: what enters the recurrence
 // Per token, in place: every q and k head becomes a unit vector, x / sqrt(sum x^2 + unit_eps), q times q_scale;
 // a[t, h, i] becomes the decay exp(-exp(a_log[h]) * softplus(a + dt_bias[h, i])); beta[t, h] = sigmoid(b[t, h]).
-__global__ void delta_prep_kernel(float* __restrict__ qk, size_t qk_stride, int n_kv, int dim, float* __restrict__ a,
+__global__ __launch_bounds__(1024) void delta_prep_kernel(float* __restrict__ qk, size_t qk_stride, int n_kv, int dim, float* __restrict__ a,
                                   size_t a_stride, const float* __restrict__ dt_bias, const float* __restrict__ a_log, int n_heads,
                                   const float* __restrict__ b_in, size_t b_stride, float* __restrict__ beta,
                                   float q_scale, float unit_eps) {
@@ -133,7 +133,9 @@ extern "C" int rb_delta_prep(float* qk, long long qk_stride, int n_kv_heads, int
   RB_REQUIRE(qk_stride >= 2LL * n_kv_heads * dim && b_stride >= n_heads && a_stride >= (long long)n_heads * dim,
              "rb_delta_prep: a row stride is too short");
   if (n_tokens == 0) return 0;
-  delta_prep_kernel<<<n_tokens, 256, 0, (hipStream_t)stream>>>(qk, (size_t)qk_stride, n_kv_heads, dim, a, (size_t)a_stride, dt_bias, a_log,
+  // a step of few tokens has few workgroups, and a token's heads are a chain of trips to memory for each wave: more waves then
+  const int threads = n_tokens < 2 * rb_compute_units() ? 1024 : 256;
+  delta_prep_kernel<<<n_tokens, threads, 0, (hipStream_t)stream>>>(qk, (size_t)qk_stride, n_kv_heads, dim, a, (size_t)a_stride, dt_bias, a_log,
                                                                n_heads, b_in, (size_t)b_stride, beta, q_scale, unit_eps);
   RB_LAUNCH_CHECK();
   return 0;
@@ -224,6 +226,7 @@ __global__ __launch_bounds__(RB_WAVE) void delta_rule_kernel(
     if (lane < CH) sb[lane] = rb;
     __syncthreads();
     if (t0 + CH < n) fetch(t0 + CH);                   // in flight while this chunk is computed
+    __builtin_amdgcn_sched_barrier(0);                 // (issued here, not where the scheduler would sink them: at their use)
     // One token: with D = diag(g) S and u = beta (v - D^T k), the read-out of the updated state is
     // (D + k u^T)^T q = D^T q + u (k . q): one pass over the decayed column gives both dot products, and a token has
     // one reduction among the RG lanes on its way instead of two.  Two partial sums each: shorter chains of additions.
