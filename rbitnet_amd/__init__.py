@@ -11,12 +11,12 @@ block), `cache` (slots, pages, state), `engine` (model, step, generation), `samp
 `csrc` (the HIP kernels).  Importing the package needs no GPU; building an Engine does.
 """
 from .errors import (CacheError, ConfigError, InferenceError, KernelError, RbitnetError, WeightError)
-from .config import LlamaConfig, load_config, register_architecture
+from .config import BagonexConfig, LlamaConfig, load_config, register_architecture
 from .engine import Engine, GenerationResult
 from .weights import write_random_model
 
 __version__ = "0.1.0"
 
-__all__ = ["Engine", "GenerationResult", "LlamaConfig", "load_config", "register_architecture",
+__all__ = ["Engine", "GenerationResult", "LlamaConfig", "BagonexConfig", "load_config", "register_architecture",
            "write_random_model", "RbitnetError", "ConfigError", "WeightError", "CacheError", "InferenceError",
            "KernelError", "__version__"]

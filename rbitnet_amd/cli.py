@@ -136,19 +136,23 @@ def cmd_inspect(args) -> int:
     if os.path.isfile(cfg_path):
         with open(cfg_path) as f:
             raw = json.load(f)
-        arch = (raw.get("architectures") or ["?"])[0]
+        from .config import architecture_of
+        try:
+            arch = architecture_of(raw)
+        except Exception:
+            arch = "?"
     print(f"safetensors arch={arch} tensors={len(names)} files={len(store.files)}")
     print(f"tensor_data_len={n_bytes} bytes")
     if raw is not None:
         from .config import load_config
-        cfg, spec = load_config(raw)
+        cfg, spec = load_config(raw, tensor_names=names, tensor_shapes={n: tuple(store.info(n)[1]) for n in names})
         fields = {k: v for k, v in vars(cfg).items() if not k.startswith("_")}
         print(f"{type(cfg).__name__}: " + " ".join(f"{k}={v!r}" for k, v in fields.items()))
         from .engine.model import expected_tensors
         from .weights.loader import resolve_names
         expected = expected_tensors(spec)
         _, missing, unexpected = resolve_names(expected, names, getattr(type(cfg), "tensor_aliases", None),
-                                               ["lm_head.weight"] if spec.head_name is None else [])
+                                               spec.optional_tensors)
         print(f"expected tensors={len(expected)} missing={len(missing)} unexpected={len(unexpected)}")
     show = min(20, len(names))
     print(f"First {show} tensors:")

@@ -57,9 +57,11 @@ def load_config(path_or_dict: Any, tensor_names: Optional[Iterable[str]] = None,
     """config.json (a folder, a file or an already parsed dict) -> (typed
     configuration, spec).  tensor_names: the names in the weight file that goes with it;
     tensor_shapes: name -> shape of the same, for a configuration that reads sizes off them."""
+    folder = None
     if isinstance(path_or_dict, dict):
         raw = path_or_dict
     else:
+        folder = path_or_dict if os.path.isdir(path_or_dict) else os.path.dirname(os.path.abspath(path_or_dict))
         path = path_or_dict
         if os.path.isdir(path):
             path = os.path.join(path, "config.json")
@@ -76,8 +78,18 @@ def load_config(path_or_dict: Any, tensor_names: Optional[Iterable[str]] = None,
     cfg = cls.from_dict(raw)
     if tensor_names is not None and hasattr(cfg, "with_tensor_names"):
         cfg = cfg.with_tensor_names(list(tensor_names))
-    if tensor_shapes is not None and hasattr(cfg, "with_tensor_shapes"):
-        cfg = cfg.with_tensor_shapes(tensor_shapes)
+    if hasattr(cfg, "with_tensor_shapes"):
+        if tensor_shapes is None and folder is not None:
+            # a configuration that reads sizes off the weights finds the file that lies beside it, if there is one
+            from ..weights.safetensors_io import WeightFolder
+            from ..errors import WeightError
+            try:
+                store = WeightFolder(folder)
+                tensor_shapes = {name: tuple(store.info(name)[1]) for name in store.names()}
+            except (WeightError, OSError):
+                tensor_shapes = None
+        if tensor_shapes is not None:
+            cfg = cfg.with_tensor_shapes(tensor_shapes)
     return cfg, cfg.to_spec()
 
 

@@ -51,8 +51,11 @@ __global__ void short_conv_kernel(const float* __restrict__ x, size_t x_stride, 
       wt[j] = j < keep ? w[(size_t)c * taps + j] : 0.f;
     }
     const float w_cur = w[(size_t)c * taps + keep];
+    float nxt = first > 0 ? x[(size_t)row0 * x_stride + c] : 0.f;
+    __builtin_amdgcn_sched_barrier(0);                       // state, weights and the first row: one trip to memory together
     for (int i = 0; i < first; ++i) {
-      const float cur = x[(size_t)(row0 + i) * x_stride + c];
+      const float cur = nxt;
+      if (i + 1 < first) nxt = x[(size_t)(row0 + i + 1) * x_stride + c];
       float acc = residual ? cur : 0.f;
       acc = fmaf(w_cur, cur, acc);
 #pragma unroll

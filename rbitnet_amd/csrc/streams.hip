@@ -143,6 +143,14 @@ __global__ __launch_bounds__(1024) void streams_layernorm_vec_kernel(
     *reinterpret_cast<float4*>(u + j) = v;
     sum += (v.x + v.y) + (v.z + v.w);
   }
+  // weight and bias of this thread's first values are asked for now, so that they arrive under the two reductions
+  const int j0 = 4 * threadIdx.x;
+  float4 w0 = make_float4(0.f, 0.f, 0.f, 0.f), b0 = w0;
+  if (j0 < width) {
+    w0 = ld4(weight + j0);
+    if (bias) b0 = ld4(bias + j0);
+  }
+  __builtin_amdgcn_sched_barrier(0);
   const float mean = block_sum(sum, scratch) / (float)width;
   float ss = 0.f;
   for (int j = 4 * threadIdx.x; j < width; j += 4 * blockDim.x) {
@@ -154,10 +162,10 @@ __global__ __launch_bounds__(1024) void streams_layernorm_vec_kernel(
   TO* orow = out + (size_t)r * width;
   for (int j = 4 * threadIdx.x; j < width; j += 4 * blockDim.x) {
     const float4 v = *reinterpret_cast<const float4*>(u + j);
-    const float4 wv = ld4(weight + j);
+    const float4 wv = j == j0 ? w0 : ld4(weight + j);
     float4 o = make_float4((v.x - mean) * f * wv.x, (v.y - mean) * f * wv.y, (v.z - mean) * f * wv.z, (v.w - mean) * f * wv.w);
     if (bias) {
-      const float4 bv = ld4(bias + j);
+      const float4 bv = j == j0 ? b0 : ld4(bias + j);
       o = make_float4(o.x + bv.x, o.y + bv.y, o.z + bv.z, o.w + bv.w);
     }
     st4(orow + j, o.x, o.y, o.z, o.w);

@@ -83,3 +83,19 @@ def test_a_layer_may_ask_the_cache_for_several_things():
     assert c.alloc_slot() == s and float(c.view(1, tables).states["delta"][s].abs().max()) == 0.0     # handed out clean
     with pytest.raises(Exception, match="twice"):
         Cache([[CacheRequest("state", state_shape=(2,)), CacheRequest("state", state_shape=(2,))]], 1, 64, torch.float32, "cpu")
+
+
+def test_command_line_writes_and_inspects_a_random_model(tmp_path, capsys):
+    import json
+    from rbitnet_amd import cli
+    cfg_path = tmp_path / "config.json"
+    cfg_path.write_text(json.dumps(CFG))
+    assert cli.main(["random", "--config", str(cfg_path), "--out", str(tmp_path / "m"), "--seed", "3"]) == 0
+    capsys.readouterr()
+    assert cli.main(["inspect", str(tmp_path / "m")]) == 0
+    out = capsys.readouterr().out
+    assert "arch=Bagonex" in out and "BagonexConfig" in out and "missing=0 unexpected=0" in out
+    # the mixing matrices of a random model start near the identity, so that the copies of the stream survive the layers
+    from rbitnet_amd.weights.safetensors_io import WeightFolder
+    mix = WeightFolder(str(tmp_path / "m")).tensor("l1.hc2.mix").float()
+    assert mix.shape == (3, 3) and float((mix - torch.eye(3)).abs().max()) < 0.2

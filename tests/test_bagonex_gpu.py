@@ -423,3 +423,39 @@ def test_long_decoding_and_greedy_generation_through_the_engine():
         assert all(g == t for g, t, c in zip(greedy, r.tokens, clear.tolist()) if c)
         assert int(clear.sum()) > 0.9 * n
     assert eng.stats["decode_tokens"] > 0 and eng.model.graph_safe
+
+
+def test_replay_and_command_line_on_a_model_of_this_design(tmp_path, capsys):
+    """The trace replay (steps from a stream of JSON lines, logits to files) and `rbitnet generate` on model B:
+    the replayed logits are the plain ones, whole and decoded, and the command line prints greedy tokens."""
+    import io
+    import numpy as np
+    from rbitnet_amd import cli
+    from rbitnet_amd.replay import replay
+    folder, oracle = _model("B")
+    eng = _engine("B", "float32", max_tokens=64 * 6, max_batch=4)
+    a, b = _tokens("B", 70, 5), _tokens("B", 9, 6)
+    lines = [json.dumps({"step": 0, "entries": [{"id": "a", "tokens": a[:66], "want": [0, 65]},
+                                                {"id": "b", "tokens": b[:8], "want": []}], "end": []}),
+             json.dumps({"step": 1, "entries": [{"id": "a", "tokens": a[66:67], "want": [0]},
+                                                {"id": "b", "tokens": b[8:9], "want": [0]}], "end": ["b"]}),
+             json.dumps({"step": 2, "entries": [{"id": "a", "tokens": a[67:], "want": [2]}], "end": ["a"]})]
+    log = io.StringIO()
+    assert replay(eng, io.StringIO("\n".join(lines) + "\n"), str(tmp_path / "out"), log=log) == 3
+    assert log.getvalue().split() == ["done", "0", "done", "1", "done", "2"]
+    wa, wb = oracle.logits(a), oracle.logits(b)
+    vocab = MODELS["B"][0]["vocab"]
+    got0 = np.fromfile(tmp_path / "out" / "0.f32", dtype="<f4").reshape(-1, vocab)
+    got1 = np.fromfile(tmp_path / "out" / "1.f32", dtype="<f4").reshape(-1, vocab)
+    got2 = np.fromfile(tmp_path / "out" / "2.f32", dtype="<f4").reshape(-1, vocab)
+    assert _close(torch.from_numpy(got0), wa[[0, 65]], "float32")
+    assert _close(torch.from_numpy(got1), torch.stack([wa[66], wb[8]]), "float32")
+    assert _close(torch.from_numpy(got2), wa[[69]], "float32")
+    assert eng.cache.live_slots == []
+    del eng
+    capsys.readouterr()
+    assert cli.main(["generate", "--model", folder, "--dtype", "float32", "--prompt-ids", ",".join(str(t) for t in b),
+                     "--max-tokens", "5", "--temperature", "0"]) == 0
+    out = capsys.readouterr().out
+    rec = json.loads(out.strip().splitlines()[-1])
+    assert len(rec["tokens"]) == 5 and rec["tokens"][0] == int(oracle.logits(b)[-1].argmax())
