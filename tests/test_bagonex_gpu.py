@@ -326,7 +326,24 @@ MODEL_B = {"architecture": "Bagonex", "vocab": 33, "width": 32, "streams": 1, "n
            "logit_softcap": 30.0, "layers": [
                _layer("channel_delta", heads=1, kv_heads=1, dim=32, vdim=32, conv=4, mlp=32),
                _layer("latent_attention", heads=1, dim=32, vdim=32, q_rank=32, kv_rank=32, scale=1.0, mlp=None)]}
-MODELS = {"A": (MODEL_A, 11), "B": (MODEL_B, 12)}
+# sizes that no kernel's fast path was made for: a width that is no multiple of 16, odd head counts, a latent of 80 and
+# one of 128 under five heads, ranks that are no multiples of 8, four copies, the first layer an attention layer,
+# two readers of one layer's latents, delta layers without a feed-forward
+MODEL_C = {"architecture": "Bagonex", "vocab": 101, "width": 72, "streams": 4, "norm": {"eps": 1e-6}, "canon": {"taps": 4},
+           "logit_softcap": 12.0, "layers": [
+               _layer("latent_attention", heads=5, dim=24, vdim=40, q_rank=44, kv_rank=128, scale=0.2, mlp=100),
+               _layer("channel_delta", heads=6, kv_heads=1, dim=48, vdim=20, conv=2, mlp=None),
+               _layer("latent_attention", heads=7, dim=8, vdim=8, q_rank=20, kv_rank=128, scale=0.35, kv_from=0, mlp=None),
+               _layer("latent_attention", heads=3, dim=40, vdim=12, q_rank=36, kv_rank=80, scale=0.15, mlp=44),
+               _layer("channel_delta", heads=3, kv_heads=3, dim=100, vdim=36, conv=5, mlp=88),
+               _layer("latent_attention", heads=2, dim=16, vdim=16, q_rank=12, kv_rank=128, scale=0.25, kv_from=0, mlp=36)]}
+# widths and ranks on the matrix cores' grid, many heads on a latent of 64 (more than a decode kernel's group takes)
+MODEL_D = {"architecture": "Bagonex", "vocab": 320, "width": 128, "streams": 2, "norm": {"eps": 1e-5}, "canon": {"taps": 3},
+           "logit_softcap": 20.0, "layers": [
+               _layer("channel_delta", heads=4, kv_heads=2, dim=64, vdim=64, conv=4, decay_rank=16, gate_rank=32, mlp=256),
+               _layer("latent_attention", heads=20, dim=16, vdim=16, q_rank=64, kv_rank=64, scale=0.25, mlp=256),
+               _layer("channel_delta", heads=2, kv_heads=2, dim=128, vdim=32, conv=4, decay_rank=8, gate_rank=8, mlp=None)]}
+MODELS = {"A": (MODEL_A, 11), "B": (MODEL_B, 12), "C": (MODEL_C, 13), "D": (MODEL_D, 14)}
 _TMP = tempfile.TemporaryDirectory(prefix="bagonex_models_")
 _MADE = {}
 
@@ -370,6 +387,36 @@ def test_model_whole_in_pieces_and_decoded(name, dtype):
             at += n
         eng.free_slot(slot)
         assert _close(torch.cat(out), want, dtype), cuts
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["C", "D"])
+def test_models_of_other_shapes_as_a_batch_in_pieces(name, dtype):
+    """Two requests of unequal lengths together: their prompts in two unequal pieces each (so that the second piece
+    reads states and latents that the first left), then token by token; against each request's plain logits."""
+    eng = _engine(name, dtype, max_tokens=64 * 8, max_batch=2)
+    oracle = _model(name)[1]
+    seqs = [_tokens(name, 150, 21), _tokens(name, 71, 22)]
+    want = [oracle.logits(s) for s in seqs]
+    slots = [eng.alloc_slot() for _ in seqs]
+    got = [[], []]
+    at = [0, 0]
+    for pieces in ([67, 3], [62, 60]):
+        logits = eng.step([(sl, s[a:a + n]) for sl, s, a, n in zip(slots, seqs, at, pieces)], "all")
+        got[0].append(logits[:pieces[0]])
+        got[1].append(logits[pieces[0]:])
+        at = [a + n for a, n in zip(at, pieces)]
+    live = [0, 1]
+    while live:
+        logits = eng.step([(slots[i], [seqs[i][at[i]]]) for i in live], "last")
+        for row, i in enumerate(live):
+            got[i].append(logits[row:row + 1])
+            at[i] += 1
+        for i in [i for i in live if at[i] >= len(seqs[i])]:
+            eng.free_slot(slots[i])
+            live.remove(i)
+    for i in range(2):
+        assert _close(torch.cat(got[i]), want[i], dtype), i
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
