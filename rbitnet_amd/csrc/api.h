@@ -171,11 +171,12 @@ int rb_short_conv(const float* x, long long x_stride, const float* w, int taps, 
 int rb_delta_prep(float* qk, long long qk_stride, int n_kv_heads, int dim, float* a, long long a_stride, const float* dt_bias, const float* a_log,
                   int n_heads, const float* b_in, long long b_stride, float* beta, float q_scale, float unit_eps, int n_tokens,
                   void* stream);
-// Per sequence b (rows cu_seqlens[b]..) and head h, token after token on state [slots, H, dim, vdim]:
+// Per sequence b (rows cu_seqlens[b]..) and head h, token after token on the state S, kept column by column as
+// [slots, H, vdim, dim]:
 //   S <- diag(g) S;  u = beta (v - S^T k);  S <- S + k u^T;  out[t, h, :] = S^T q      (head h reads q/k head h / (H / Hk))
 int rb_delta_rule(const float* q, const float* k, long long qk_stride, const float* v, long long v_stride, const float* g,
                   long long g_stride, const float* beta, float* state, const int32_t* cu_seqlens, const int32_t* slots, float* out, int n_seqs,
-                  int n_heads, int n_kv_heads, int dim, int vdim, void* stream);
+                  int n_tokens, int n_heads, int n_kv_heads, int dim, int vdim, void* stream);
 // out[t, h, :] = o / sqrt(mean(o^2) + eps) * weight[vdim] * sigmoid(gate[t * gate_stride + h * vdim + :])
 int rb_gated_rmsnorm(const float* o, const float* weight, const float* gate, long long gate_stride, float eps, void* out,
                      int out_dtype, int n_tokens, int n_heads, int vdim, void* stream);

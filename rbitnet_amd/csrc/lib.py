@@ -158,7 +158,7 @@ class Kernels:
             "rb_tanh_cap": [_P, _F, _L, _P],
             "rb_short_conv": [_P, _L, _P, _I, _P, _P, _P, _P, _P, _P, _L, _I, _I, _I, _I, _I, _I, _P],
             "rb_delta_prep": [_P, _L, _I, _I, _P, _L, _P, _P, _I, _P, _L, _P, _F, _F, _I, _P],
-            "rb_delta_rule": [_P, _P, _L, _P, _L, _P, _L, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _P],
+            "rb_delta_rule": [_P, _P, _L, _P, _L, _P, _L, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P],
             "rb_gated_rmsnorm": [_P, _P, _P, _L, _F, _P, _I, _I, _I, _I, _P],
             "rb_latent_norm_store": [_P, _L, _I, _P, _P, _I, _I, _P, _P, _I, _P, _P, _P, _I, _F, _I, _P],
             "rb_heads_linear": [_P, _I, _P, _I, _P, _I, _I, _I, _I, _I, _P],
@@ -550,7 +550,8 @@ class Kernels:
 
     def delta_rule(self, qkv: torch.Tensor, n_kv: int, dim: int, n_heads: int, vdim: int, g: torch.Tensor,
                    beta: torch.Tensor, state: torch.Tensor, ctx, out: torch.Tensor) -> None:
-        """qkv [T, >= (2 Hk dim + H vdim)] float32: q heads, k heads, v heads; state [slots, H, dim, vdim] float32."""
+        """qkv [T, >= (2 Hk dim + H vdim)] float32: q heads, k heads, v heads; state [slots, H, vdim, dim] float32 (the
+        matrix S [dim, vdim] of a head, kept column by column)."""
         n, width = qkv.shape
         _check(qkv, "qkv", torch.float32)
         if width < 2 * n_kv * dim + n_heads * vdim:
@@ -560,14 +561,14 @@ class Kernels:
             raise KernelError("delta_rule: rows of g too short for the decays")
         _check(beta, "beta", torch.float32, (n, n_heads))
         _check(state, "state", torch.float32)
-        if tuple(state.shape[1:]) != (n_heads, dim, vdim):
-            raise KernelError(f"delta_rule: state of shape {tuple(state.shape)}, expected [*, {n_heads}, {dim}, {vdim}]")
+        if tuple(state.shape[1:]) != (n_heads, vdim, dim):
+            raise KernelError(f"delta_rule: state of shape {tuple(state.shape)}, expected [*, {n_heads}, {vdim}, {dim}]")
         _check(out, "out", torch.float32, (n, n_heads * vdim))
         if ctx.n_tokens != n:
             raise KernelError("delta_rule: the step's tokens and the rows differ")
         base = qkv.data_ptr()
         self._ok(self._lib.rb_delta_rule(base, base + 4 * n_kv * dim, width, base + 8 * n_kv * dim, width, _ptr(g), g.shape[1], _ptr(beta),
-                                         _ptr(state), _ptr(ctx.cu_seqlens), _ptr(ctx.slots), _ptr(out), ctx.n_seqs, n_heads,
+                                         _ptr(state), _ptr(ctx.cu_seqlens), _ptr(ctx.slots), _ptr(out), ctx.n_seqs, n, n_heads,
                                          n_kv, dim, vdim, self._stream()))
 
     def gated_rmsnorm(self, o: torch.Tensor, weight: torch.Tensor, gate: torch.Tensor, gate_col: int, eps: float,

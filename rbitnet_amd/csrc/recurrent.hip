@@ -184,12 +184,27 @@ __global__ __launch_bounds__(RB_WAVE) void delta_rule_kernel(
   const bool on = col < vdim;
   const int kvh = h / (n_heads / n_kv);
   const int row0 = cu_seqlens[b], n = cu_seqlens[b + 1] - row0;
-  float* S = state + (((size_t)slots[b] * n_heads + h) * dim) * vdim;
+  // the state is kept column by column, [slots, H, vdim, dim]: a lane's rows are DKL numbers in a row and a wave's
+  // columns one piece of memory (with S as rows a wave of four columns used a quarter of every line it touched)
+  float* S = state + (((size_t)slots[b] * n_heads + h) * vdim + (on ? col : 0)) * dim;
   float s[DKL];
+  const bool quads = dim % 4 == 0 && DKL % 4 == 0 && (reinterpret_cast<uintptr_t>(state) & 15) == 0;
+  if (quads) {
 #pragma unroll
-  for (int i = 0; i < DKL; ++i) {
-    const int r = rg * DKL + i;
-    s[i] = (on && r < dim) ? S[(size_t)r * vdim + col] : 0.f;
+    for (int i = 0; i < DKL; i += 4) {
+      const int r = rg * DKL + i;
+      const float4 v4 = (on && r < dim) ? *reinterpret_cast<const float4*>(S + r) : make_float4(0.f, 0.f, 0.f, 0.f);
+      s[i] = v4.x;
+      s[i + 1] = v4.y;
+      s[i + 2] = v4.z;
+      s[i + 3] = v4.w;
+    }
+  } else {
+#pragma unroll
+    for (int i = 0; i < DKL; ++i) {
+      const int r = rg * DKL + i;
+      s[i] = (on && r < dim) ? S[r] : 0.f;
+    }
   }
   float rq[NQ], rk[NQ], rgt[NQ], rv[NV], rb = 0.f;
   auto fetch = [&](int t0) {
@@ -271,10 +286,18 @@ __global__ __launch_bounds__(RB_WAVE) void delta_rule_kernel(
       if (col0 + c < vdim) out[((size_t)(row0 + t0 + tt) * n_heads + h) * vdim + col0 + c] = so[tt][c];
     }
   }
+  if (quads) {
 #pragma unroll
-  for (int i = 0; i < DKL; ++i) {
-    const int r = rg * DKL + i;
-    if (on && r < dim) S[(size_t)r * vdim + col] = s[i];
+    for (int i = 0; i < DKL; i += 4) {
+      const int r = rg * DKL + i;
+      if (on && r < dim) *reinterpret_cast<float4*>(S + r) = make_float4(s[i], s[i + 1], s[i + 2], s[i + 3]);
+    }
+  } else {
+#pragma unroll
+    for (int i = 0; i < DKL; ++i) {
+      const int r = rg * DKL + i;
+      if (on && r < dim) S[r] = s[i];
+    }
   }
 }
 
@@ -284,7 +307,7 @@ static void launch_delta_rule(const float* q, const float* k, size_t qk_stride, 
                               const int32_t* slots, float* out, int n_seqs, int n_heads, int n_kv, int dim, int vdim,
                               hipStream_t s) {
   constexpr int COLS = RB_WAVE / RG;
-  static_assert((DKL * RG * CH) % RB_WAVE == 0 && CH <= RB_WAVE && DKL % 2 == 0, "a chunk's values are dealt evenly to the lanes");
+  static_assert((DKL * RG * CH) % RB_WAVE == 0 && CH <= RB_WAVE && DKL % 4 == 0, "a chunk's values are dealt evenly to the lanes");
   dim3 grid(n_seqs, n_heads, (vdim + COLS - 1) / COLS);
   delta_rule_kernel<DKL, RG, CH><<<grid, RB_WAVE, 0, s>>>(q, k, qk_stride, v, v_stride, g, g_stride, beta, state, cu_seqlens,
                                                           slots, out, n_heads, n_kv, dim, vdim);
@@ -292,10 +315,10 @@ static void launch_delta_rule(const float* q, const float* k, size_t qk_stride, 
 
 extern "C" int rb_delta_rule(const float* q, const float* k, long long qk_stride, const float* v, long long v_stride,
                              const float* g, long long g_stride, const float* beta, float* state, const int32_t* cu_seqlens,
-                             const int32_t* slots, float* out, int n_seqs, int n_heads, int n_kv_heads, int dim, int vdim,
-                             void* stream) {
-  RB_RECORDED(rb_delta_rule(q, k, qk_stride, v, v_stride, g, g_stride, beta, state, cu_seqlens, slots, out, n_seqs, n_heads,
-                            n_kv_heads, dim, vdim, stream));
+                             const int32_t* slots, float* out, int n_seqs, int n_tokens, int n_heads, int n_kv_heads, int dim,
+                             int vdim, void* stream) {
+  RB_RECORDED(rb_delta_rule(q, k, qk_stride, v, v_stride, g, g_stride, beta, state, cu_seqlens, slots, out, n_seqs, n_tokens,
+                            n_heads, n_kv_heads, dim, vdim, stream));
   RB_REQUIRE(n_seqs >= 0 && n_heads > 0 && n_kv_heads > 0 && n_heads % n_kv_heads == 0 && dim > 0 && vdim > 0,
              "rb_delta_rule: bad sizes H=%d Hk=%d dim=%d vdim=%d", n_heads, n_kv_heads, dim, vdim);
   RB_REQUIRE(g_stride >= (long long)n_heads * dim, "rb_delta_rule: the decays' row stride is too short");
@@ -304,8 +327,19 @@ extern "C" int rb_delta_rule(const float* q, const float* k, long long qk_stride
   if (n_seqs == 0) return 0;
   hipStream_t s = (hipStream_t)stream;
   const size_t qs = (size_t)qk_stride, vs = (size_t)v_stride;
-#define DR_GO(DKL, RG, CH) \
-  launch_delta_rule<DKL, RG, CH>(q, k, qs, v, vs, g, (size_t)g_stride, beta, state, cu_seqlens, slots, out, n_seqs, n_heads, n_kv_heads, dim, vdim, s)
+  // a step of one token per sequence (n_tokens == n_seqs) stages chunks of as few tokens as deal evenly to the lanes:
+  // the machinery of a chunk of 16 would cost it several times its arithmetic
+  const bool single = n_tokens <= n_seqs;
+#define DR_GO(DKL, RG, CH)                                                                                                  \
+  do {                                                                                                                      \
+    constexpr int CH1 = (DKL * RG >= RB_WAVE) ? 1 : RB_WAVE / (DKL * RG);                                                   \
+    if (single)                                                                                                             \
+      launch_delta_rule<DKL, RG, CH1>(q, k, qs, v, vs, g, (size_t)g_stride, beta, state, cu_seqlens, slots, out, n_seqs,   \
+                                      n_heads, n_kv_heads, dim, vdim, s);                                                   \
+    else                                                                                                                    \
+      launch_delta_rule<DKL, RG, CH>(q, k, qs, v, vs, g, (size_t)g_stride, beta, state, cu_seqlens, slots, out, n_seqs,    \
+                                     n_heads, n_kv_heads, dim, vdim, s);                                                    \
+  } while (0)
   // Rows of a column over RG lanes, chunks as long as the registers that hold the next one allow.  A token's time is
   // its lane's share of the column, so while the waves do not fill the GPU's SIMDs a column goes to more lanes
   // (more and shorter waves); once they do, fewer lanes per column save the moves between them.

@@ -12,7 +12,8 @@ Per token, with h the mixer's input:
 
 In float32: everything from the unit vectors on (decays, beta, the recurrence, the read-out norm and its gate); the
 projections and the convolution's inputs are float32 sums of products in the compute dtype.  The state and the
-convolution's last taps - 1 inputs live in the cache (`view.states["delta"]`, `view.states["conv"]`).
+convolution's last taps - 1 inputs live in the cache (`view.states["delta"]`, kept column by column as
+[slots, heads, vdim, dim], and `view.states["conv"]`).
 
 Parameters: heads, kv_heads, dim, vdim, conv (taps), eps (of the read-out norm), unit_eps (1e-6), low-rank sizes come
 from the tensors' declared shapes: decay_rank, gate_rank.  names: the tensors below the layer's prefix.
@@ -97,7 +98,7 @@ class ChannelDelta(Part):
         self.w_o = pack_rows(lib, [(o, 0, None, None)], o.shape[0], o.shape[1], o.dtype, o.device, allowed)
 
     def cache_requests(self) -> List[CacheRequest]:
-        out = [CacheRequest("state", state_shape=(self.heads, self.dim, self.vdim), state_init=0.0, name="delta")]
+        out = [CacheRequest("state", state_shape=(self.heads, self.vdim, self.dim), state_init=0.0, name="delta")]
         conv = self.conv.cache_request("conv")
         return out + ([conv] if conv else [])
 

@@ -65,7 +65,7 @@ def test_a_layer_may_ask_the_cache_for_several_things():
     """Latents as keys and values at once (no second set of pages), two named states beside them, and a reader."""
     reqs = [[CacheRequest("kv", heads=1, head_dim=16, values=False, name="latent"),
              CacheRequest("state", state_shape=(1, 32), name="input_conv")],
-            [CacheRequest("state", state_shape=(4, 8, 12), name="delta"), CacheRequest("state", state_shape=(2, 40), name="conv"),
+            [CacheRequest("state", state_shape=(4, 12, 8), name="delta"), CacheRequest("state", state_shape=(2, 40), name="conv"),
              CacheRequest("state", state_shape=(1, 32), name="input_conv")],
             [CacheRequest("state", state_shape=(1, 32), name="input_conv")]]
     c = Cache(reqs, n_slots=2, max_tokens=128, dtype=torch.float32, device="cpu", readers={2: 0})
@@ -75,7 +75,7 @@ def test_a_layer_may_ask_the_cache_for_several_things():
     v0, v1, v2 = (c.view(l, tables) for l in range(3))
     assert v0.k_pages.shape == (3, 1, 64, 16) and v0.v_pages.data_ptr() == v0.k_pages.data_ptr()
     assert v2.k_pages.data_ptr() == v0.k_pages.data_ptr() and set(v2.states) == {"input_conv"}
-    assert v1.states["delta"].shape == (3, 4, 8, 12) and v1.states["conv"].shape == (3, 2, 40) and v1.k_pages is None
+    assert v1.states["delta"].shape == (3, 4, 12, 8) and v1.states["conv"].shape == (3, 2, 40) and v1.k_pages is None
     assert v0.states["input_conv"].data_ptr() != v2.states["input_conv"].data_ptr()       # a layer's own
     v1.states["delta"][s] = 3.0
     c.commit([s], [70])

@@ -232,7 +232,7 @@ def test_delta_recurrence_kernel_keeps_what_was_written_long_ago(lib):
 
 def P_REQ(h, dk, dv):
     from rbitnet_amd.parts import CacheRequest
-    return CacheRequest("state", state_shape=(h, dk, dv), state_init=0.0, name="delta")
+    return CacheRequest("state", state_shape=(h, dv, dk), state_init=0.0, name="delta")      # S of a head, column by column
 
 
 # ---------------------------------------------------------------------------- latent attention
