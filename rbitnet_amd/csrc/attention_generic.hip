@@ -1,5 +1,5 @@
 // Causal attention of each token over its sequence's paged cache: any even head_dim up to
-// 256, any number of heads and groups, float32 or bfloat16 storage, float32 arithmetic
+// 512, any number of heads and groups, float32 or bfloat16 storage, float32 arithmetic
 // throughout (scores, softmax, weighted sum).  One workgroup per (token, query head): one wave
 // when the step has many tokens, up to 8 waves that share the pages of the context and merge
 // their running softmax states through LDS when it has few (a decode step of 8 sequences and
@@ -15,7 +15,8 @@
 #include "api.h"
 #include "common.h"
 
-#define AG_MAX_D 256
+#define AG_MAX_D 512
+#define AG_MAX_D_VEC 256      // the 16-byte kernel deals a row's quads to the lanes of one wave
 
 #define AG_MAX_WAVES 8
 
@@ -288,7 +289,7 @@ extern "C" int rb_attention_generic_sinks(const void* q, const void* k_pages, co
   int n_waves = 1;
   while (n_waves < AG_MAX_WAVES && (long long)n_tokens * n_heads * n_waves < 8LL * rb_compute_units()) n_waves *= 2;
   const int threads = RB_WAVE * n_waves;
-  if (head_dim % 4 == 0 && g_attention_vec) {
+  if (head_dim % 4 == 0 && head_dim <= AG_MAX_D_VEC && g_attention_vec) {
     int group_lanes = 1;
     while (group_lanes < head_dim / 4) group_lanes *= 2;
     RB_REQUIRE(dtype == RB_F32 || dtype == RB_BF16, "rb_attention_generic: unknown dtype %d", dtype);

@@ -28,7 +28,7 @@ from .linear import linear, pack_rows
 
 DEFAULT_NAMES = {"dq": "dq", "dq_norm": "dq.norm", "uq": "uq", "dkv": "dkv", "dkv_norm": "dkv.norm", "uk": "uk", "uv": "uv",
                  "sink": "sink", "o": "o"}
-MAX_RANK = 256             # the attention kernel's largest head size
+MAX_RANK = 512             # the attention kernel's largest head size
 _MATRIX_CORE_RANKS = (64, 128)     # latents of these sizes in bfloat16 go through the matrix-core attention kernels
 _DECODE_MAX_HEADS = 16             # query heads on one key/value head that the matrix-core decode kernel takes
 
