@@ -456,11 +456,14 @@ def test_long_decoding_and_greedy_generation_through_the_engine():
     """Greedy generation of 150 tokens through `Engine.generate` (its scheduler, its captured decode step) gives the
     plain implementation's greedy tokens, for a batch of three unequal prompts; the logits of the last decode step are
     the plain ones."""
-    eng = _engine("A", "float32", max_tokens=64 * 12, max_batch=4)
+    eng = _engine("A", "float32", max_tokens=64 * 16, max_batch=5)
     oracle = _model("A")[1]
-    prompts = [_tokens("A", n, 3) for n in (5, 70, 1)]
-    results = eng.generate(prompts, max_tokens=[150, 40, 90], temperature=0.0)
-    for p, r, n in zip(prompts, results, (150, 40, 90)):
+    # five requests: a captured step for five runs in the one made for six, whose sixth row is an idle sequence in the
+    # cache's spare slot and page; as requests end, the steps for four, three, two and one follow
+    limits = (150, 40, 90, 12, 25)
+    prompts = [_tokens("A", n, 3) for n in (5, 70, 1, 33, 64)]
+    results = eng.generate(prompts, max_tokens=list(limits), temperature=0.0)
+    for p, r, n in zip(prompts, results, limits):
         assert len(r.tokens) == n and r.finish_reason == "length"
         seq = list(p) + r.tokens
         logits = oracle.logits(seq[:-1])
