@@ -66,6 +66,12 @@ long long rb_gemm_workspace_floats(int m, int n, int k, int epilogue);
 int rb_gemm_bf16(const void* a, const void* w, int w_layout, void* c, int dtype_out, int epilogue, int m, int n, int k,
                  float* workspace, void* stream);
 
+// rb_gemm_bf16 with an activation on the way out (epilogue 0 only): act holds xIELU's two numbers (p, q), and
+// C = xIELU(A W^T) with xIELU(z) = softplus(p) z^2 + z/2 for z > 0, (1/2 + softplus(q)) (exp(z) - 1 - z) + z/2 otherwise,
+// applied to the float32 sums before they are stored.  act null: rb_gemm_bf16.
+int rb_gemm_bf16_act(const void* a, const void* w, int w_layout, void* c, int dtype_out, int epilogue, const float* act,
+                     int m, int n, int k, float* workspace, void* stream);
+
 // The plain product (float32, epilogue 0) as the terms that the K slices of its kernel computed:
 // terms [rb_gemm_bf16_terms_count(m, n, k), M, N], to be added up in their order.  One term is
 // the product itself.  For a caller that adds them to something else anyway.

@@ -110,6 +110,23 @@ __device__ __forceinline__ void rotate_pair(float x0, float x1, float c, float s
   y1 = __fmaf_rn(x0, s, __fmul_rn(x1, c));
 }
 
+// ---------------------------------------------------------------- xIELU
+// act(z) = softplus(p) z^2 + z / 2 for z > 0, (1/2 + softplus(q)) (exp(z) - 1 - z) + z / 2 otherwise; (p, q) are two
+// numbers of the model.  xielu_pair turns them into the two factors once; xielu_value applies them.
+struct XieluPair {
+  float ap, an;
+};
+__device__ __forceinline__ XieluPair xielu_pair(const float* __restrict__ act) {
+  const float p = act[0], q = act[1];
+  XieluPair r;
+  r.ap = p > 20.0f ? p : log1pf(expf(p));
+  r.an = 0.5f + (q > 20.0f ? q : log1pf(expf(q)));
+  return r;
+}
+__device__ __forceinline__ float xielu_value(float v, float ap, float an) {
+  return v > 0.f ? fmaf(ap * v, v, 0.5f * v) : fmaf(an, expm1f(v) - v, 0.5f * v);
+}
+
 // ---------------------------------------------------------------- terms of a product
 // A product whose K was cut into slices may be left as its slices' sums, `stride` floats
 // apart: p[0] + p[stride] + ... in that order (the order in which the product's own kernel

@@ -32,6 +32,7 @@ struct GemmAfter {
   bf16_t* gained;
   float* squares;
   bool w_frag;
+  const float* act = nullptr;      // epilogue 0: the two numbers of xIELU, applied to the sums before they are stored (null: none)
 };
 
 // at most 64 tokens, any K % 8 == 0: W streamed straight into MFMA operands (gemm_skinny.hip);
@@ -47,4 +48,4 @@ bool gemm_resident_try(const GemmTokens& x, const bf16_t* w, void* c, int dtype_
 // slices it will use; more than 1 needs parts * m * n floats of workspace.
 int gemm_tiled_parts(int m, int n, int k, int epilogue);
 int gemm_tiled_launch(const bf16_t* x, const bf16_t* w, bool w_frag, void* c, float* workspace, int dtype_out,
-                      int epilogue, int m, int n, int k, hipStream_t s);
+                      int epilogue, int m, int n, int k, hipStream_t s, const float* act = nullptr);

@@ -44,7 +44,15 @@ static bool layout_ok(int w_layout, int n, int k) {
 
 extern "C" int rb_gemm_bf16(const void* a, const void* w, int w_layout, void* c, int dtype_out, int epilogue, int m,
                             int n, int k, float* workspace, void* stream) {
-  RB_RECORDED(rb_gemm_bf16(a, w, w_layout, c, dtype_out, epilogue, m, n, k, workspace, stream));
+  return rb_gemm_bf16_act(a, w, w_layout, c, dtype_out, epilogue, nullptr, m, n, k, workspace, stream);
+}
+
+// rb_gemm_bf16 with an activation on the way out: act (epilogue 0 only; null: none) holds xIELU's two numbers, and
+// C = xIELU(A W^T), applied to the float32 sums before they are stored.
+extern "C" int rb_gemm_bf16_act(const void* a, const void* w, int w_layout, void* c, int dtype_out, int epilogue,
+                                const float* act, int m, int n, int k, float* workspace, void* stream) {
+  RB_RECORDED(rb_gemm_bf16_act(a, w, w_layout, c, dtype_out, epilogue, act, m, n, k, workspace, stream));
+  RB_REQUIRE(act == nullptr || epilogue == 0, "rb_gemm_bf16: an activation goes with epilogue 0, not %d", epilogue);
   RB_REQUIRE(m >= 0 && n > 0 && k > 0, "rb_gemm_bf16: bad sizes M=%d N=%d K=%d", m, n, k);
   RB_REQUIRE(layout_ok(w_layout, n, k), "rb_gemm_bf16: W layout %d with N=%d K=%d (fragment-major needs N %% 16 == 0, K %% 64 == 0)",
              w_layout, n, k);
@@ -58,10 +66,10 @@ extern "C" int rb_gemm_bf16(const void* a, const void* w, int w_layout, void* c,
   const bf16_t* wa = (const bf16_t*)w;
   int rc = 0;
   if (tiled_parts(m, n, k, epilogue) >= 1) {
-    rc = gemm_tiled_launch(xa, wa, w_layout == 1, c, workspace, dtype_out, epilogue, m, n, k, s);
+    rc = gemm_tiled_launch(xa, wa, w_layout == 1, c, workspace, dtype_out, epilogue, m, n, k, s, act);
   } else {
     const GemmTokens x = {xa, nullptr, 0.f, nullptr};
-    const GemmAfter after = {epilogue, nullptr, nullptr, nullptr, w_layout == 1};
+    const GemmAfter after = {epilogue, nullptr, nullptr, nullptr, w_layout == 1, act};
     rc = launch_few_tokens(x, wa, c, dtype_out, after, m, n, k, s);
   }
   if (rc) return rc;

@@ -31,6 +31,7 @@ struct FoldArgs {
   bf16_t* gained;               // epilogue 3: [M, N]
   float* squares_out;           // epilogue 3: [M, ceil(N / 16)]
   int w_frag;                   // W is stored fragment-major (see gemm_internal.h)
+  const float* act;             // epilogue 0: xIELU's two numbers, applied to the sums before they are stored; null: none
 };
 
 // What a lane does with its 4 consecutive sums of token mm, columns nn.. (epilogues 0, 2, 3).
@@ -42,12 +43,15 @@ __device__ __forceinline__ void store_sums(TO* __restrict__ c, const f32x4_t& su
                                            const FoldArgs& fa) {
   const bool row_ok = mm < m;
   float sq = 0.f;
+  XieluPair xa = {0.f, 0.f};
+  if (EPI == 0 && fa.act) xa = xielu_pair(fa.act);
   if (row_ok) {
     TO* dst = c + (size_t)mm * n + nn;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       if (nn + i >= n) continue;
-      const float v = EPI >= 2 ? before[i] + sums[i] : sums[i];
+      float v = EPI >= 2 ? before[i] + sums[i] : sums[i];
+      if (EPI == 0 && fa.act) v = xielu_value(v, xa.ap, xa.an);
       Num<TO>::store(dst + i, v);
       if (EPI == 3) {
         sq += v * v;
@@ -346,7 +350,8 @@ extern "C" void rb_tune(int r, int waves) {       // experiments only; 0 = the b
 }
 
 static FoldArgs fold_args(const GemmTokens& x, const GemmAfter& after) {
-  return FoldArgs{x.squares, x.rows, x.eps, after.gain, after.gained, after.squares, after.w_frag ? 1 : 0};
+  return FoldArgs{x.squares, x.rows, x.eps, after.gain, after.gained, after.squares, after.w_frag ? 1 : 0,
+                  after.epilogue == 0 ? after.act : nullptr};
 }
 
 template <int MB, int R, int U, bool FAST, int EPI, typename TO, bool SCALED>

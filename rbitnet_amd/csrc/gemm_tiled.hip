@@ -15,11 +15,16 @@
 // Adds up the [M, N] slabs of partial sums that the K slices of a product wrote, in slice
 // order (the same order whatever else runs), and converts to the output type.
 template <typename TO>
-__global__ void gemm_sum_slabs_kernel(const float* __restrict__ slabs, TO* __restrict__ c, int parts, size_t count) {
+__global__ void gemm_sum_slabs_kernel(const float* __restrict__ slabs, TO* __restrict__ c, int parts, size_t count,
+                                      const float* __restrict__ act) {
   const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= count) return;
   float v = 0.f;
   for (int p = 0; p < parts; ++p) v += slabs[(size_t)p * count + i];
+  if (act) {                               // an activation belongs to the whole sum: here, not in the slices
+    const XieluPair a = xielu_pair(act);
+    v = xielu_value(v, a.ap, a.an);
+  }
   Num<TO>::store(c + i, v);
 }
 
@@ -49,7 +54,8 @@ __device__ __forceinline__ bool tile_of_workgroup(int m_tiles, int n_tiles, int*
 // `slab`, the sums go to that slice's [M, N] slab instead, to be added up later in a fixed order.
 template <int EPI, typename TO>
 __device__ __forceinline__ void store_piece(const f32x16_t& acc, TO* __restrict__ c, float* __restrict__ slab,
-                                            int first_row, int l32, int mbase, int m, int n) {
+                                            int first_row, int l32, int mbase, int m, int n, bool has_act = false,
+                                            float ap = 0.f, float an = 0.f) {
   if (EPI == 0) {
     const int nn = first_row + l32;
     if (nn >= n) return;
@@ -58,7 +64,7 @@ __device__ __forceinline__ void store_piece(const f32x16_t& acc, TO* __restrict_
       const int mm = mbase + 8 * (e / 4) + (e % 4);
       if (mm >= m) continue;
       if (slab) slab[(size_t)mm * n + nn] = acc[e];
-      else Num<TO>::store(c + (size_t)mm * n + nn, acc[e]);
+      else Num<TO>::store(c + (size_t)mm * n + nn, has_act ? xielu_value(acc[e], ap, an) : acc[e]);
     }
   } else {
     // gate rows in lanes 0..15 of a half wave, up rows in lanes 16..31: the two halves swap what
@@ -85,7 +91,8 @@ __device__ __forceinline__ void store_piece(const f32x16_t& acc, TO* __restrict_
 template <int BN, int BM, int WN, int WM, int P, int EPI, bool KTAIL, typename TO>
 __global__ __launch_bounds__(64 * (BN / WN) * (BM / WM)) void gemm_tiled_kernel(const bf16_t* __restrict__ x,
                                                          const bf16_t* __restrict__ w, TO* __restrict__ c,
-                                                         int m, int n, int k, int m_tiles, int n_tiles) {
+                                                         int m, int n, int k, int m_tiles, int n_tiles,
+                                                         const float* __restrict__ act) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   constexpr int TN = WN / 32, TM = WM / 32;
   constexpr int WAVES_N = BN / WN;
@@ -233,11 +240,14 @@ __global__ __launch_bounds__(64 * (BN / WN) * (BM / WM)) void gemm_tiled_kernel(
   }
 
   // ---- lane holds, per (i, j): W row n0 + wn0 + 32 i + l32, tokens base + 8 (e / 4) + 4 g + e % 4
+  const bool has_act = EPI == 0 && act != nullptr;
+  XieluPair xa = {0.f, 0.f};
+  if (has_act) xa = xielu_pair(act);
 #pragma unroll
   for (int i = 0; i < TN; ++i)
 #pragma unroll
     for (int j = 0; j < TM; ++j)
-      store_piece<EPI, TO>(acc[i][j], c, nullptr, n0 + wn0 + 32 * i, l32, m0 + wm0 + 32 * j + 4 * g, m, n);
+      store_piece<EPI, TO>(acc[i][j], c, nullptr, n0 + wn0 + 32 * i, l32, m0 + wm0 + 32 * j + 4 * g, m, n, has_act, xa.ap, xa.an);
 }
 
 // ---------------------------------------------------------------------------------------
@@ -257,7 +267,7 @@ template <int BN, int BM, int WN, int WM, int BK, int S, int EPI, typename TO, b
 __global__ __launch_bounds__(64 * (BN / WN) * (BM / WM)) void gemm_dma_kernel(const bf16_t* __restrict__ x,
                                                        const bf16_t* __restrict__ w, TO* __restrict__ c,
                                                        float* __restrict__ slabs, int m, int n, int k, int m_tiles,
-                                                       int n_tiles, int k_tiles) {
+                                                       int n_tiles, int k_tiles, const float* __restrict__ act) {
   extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
   constexpr int TN = WN / 32, TM = WM / 32;
   constexpr int WAVES_N = BN / WN;
@@ -528,16 +538,19 @@ __global__ __launch_bounds__(64 * (BN / WN) * (BM / WM)) void gemm_dma_kernel(co
     return;
   }
   float* slab = slabs ? slabs + (size_t)blockIdx.y * m * n : nullptr;      // this slice of K's partial sums
+  const bool has_act = EPI == 0 && act != nullptr && slab == nullptr;      // slices leave the activation to the sum of the slabs
+  XieluPair xa = {0.f, 0.f};
+  if (has_act) xa = xielu_pair(act);
 #pragma unroll
   for (int i = 0; i < TN; ++i)
 #pragma unroll
     for (int j = 0; j < TM; ++j)
-      store_piece<EPI, TO>(acc[i][j], c, slab, n0 + wn0 + 32 * i, l32, m0 + wm0 + 32 * j + 4 * g, m, n);
+      store_piece<EPI, TO>(acc[i][j], c, slab, n0 + wn0 + 32 * i, l32, m0 + wm0 + 32 * j + 4 * g, m, n, has_act, xa.ap, xa.an);
 }
 
 template <int BN, int BM, int WN, int WM, int BK, int S, int EPI, typename TO, bool WF>
 static int launch_dma_cfg(const bf16_t* x, const bf16_t* w, void* c, int m, int n, int k, hipStream_t s,
-                          int parts = 1, float* slabs = nullptr) {
+                          int parts = 1, float* slabs = nullptr, const float* act = nullptr) {
   const int m_tiles = (m + BM - 1) / BM, n_tiles = (n + BN - 1) / BN;
   RB_REQUIRE(parts >= 1 && (k / BK) % parts == 0 && (parts == 1 || (slabs && EPI == 0)),
              "rb_gemm_bf16: internal: bad K split %d", parts);
@@ -557,18 +570,20 @@ static int launch_dma_cfg(const bf16_t* x, const bf16_t* w, void* c, int m, int 
     configured = true;
   }
   const dim3 grid((unsigned)((tiles + 7) / 8 * 8), (unsigned)parts);
+  RB_REQUIRE(act == nullptr || (EPI == 0 && c != nullptr), "rb_gemm_bf16: internal: an activation goes with epilogue 0 and an output");
   kern<<<grid, 64 * (BN / WN) * (BM / WM), lds, s>>>(x, w, (TO*)c, parts > 1 ? slabs : nullptr, m, n, k, m_tiles,
-                                                      n_tiles, k / BK / parts);
+                                                      n_tiles, k / BK / parts, act);
   if (parts > 1 && c != nullptr) {      // without c the caller adds the slabs up itself
     const size_t count = (size_t)m * n;
-    gemm_sum_slabs_kernel<TO><<<(unsigned)((count + 255) / 256), 256, 0, s>>>(slabs, (TO*)c, parts, count);
+    gemm_sum_slabs_kernel<TO><<<(unsigned)((count + 255) / 256), 256, 0, s>>>(slabs, (TO*)c, parts, count, act);
   }
   return 0;
 }
 
 
 template <int BN, int BM, int WN, int WM, int P, int EPI, typename TO>
-static int launch_tiled_cfg(const bf16_t* x, const bf16_t* w, void* c, int m, int n, int k, hipStream_t s) {
+static int launch_tiled_cfg(const bf16_t* x, const bf16_t* w, void* c, int m, int n, int k, hipStream_t s,
+                            const float* act = nullptr) {
   const int m_tiles = (m + BM - 1) / BM, n_tiles = (n + BN - 1) / BN;
   const long long tiles = (long long)m_tiles * n_tiles;
   RB_REQUIRE(tiles < (1LL << 30), "rb_gemm_bf16: too many tiles");
@@ -584,7 +599,7 @@ static int launch_tiled_cfg(const bf16_t* x, const bf16_t* w, void* c, int m, in
     configured[tail] = true;
   }
   const int grid = (int)((tiles + 7) / 8 * 8);
-  kern<<<grid, 64 * (BN / WN) * (BM / WM), lds, s>>>(x, w, (TO*)c, m, n, k, m_tiles, n_tiles);
+  kern<<<grid, 64 * (BN / WN) * (BM / WM), lds, s>>>(x, w, (TO*)c, m, n, k, m_tiles, n_tiles, EPI == 0 ? act : nullptr);
   return 0;
 }
 
@@ -703,28 +718,28 @@ static TilePlan plan_tiles(int m, int n, int k, int epilogue) {
 
 template <int EPI, typename TO, bool WF>
 static int launch_planned(const bf16_t* x, const bf16_t* w, void* c, float* workspace, int m, int n, int k,
-                          hipStream_t s) {
+                          hipStream_t s, const float* act) {
   const TilePlan plan = plan_tiles(m, n, k, EPI);
   RB_REQUIRE(plan.cfg != 0, "rb_gemm_bf16: internal: M=%d N=%d K=%d is not a product for the tiled kernels", m, n, k);
   RB_REQUIRE(plan.parts == 1 || workspace != nullptr, "rb_gemm_bf16: M=%d N=%d K=%d needs a workspace of %lld floats",
              m, n, k, (long long)plan.parts * m * n);
   const int p = plan.parts;
   switch (plan.cfg) {
-    case 8: return launch_dma_cfg<256, 128, 64, 64, 64, 3, EPI, TO, WF>(x, w, c, m, n, k, s, p, workspace);
-    case 9: return launch_dma_cfg<320, 256, 160, 64, 64, 2, EPI, TO, WF>(x, w, c, m, n, k, s, p, workspace);
-    case 7: return launch_dma_cfg<128, 64, 32, 64, 64, 3, EPI, TO, WF>(x, w, c, m, n, k, s, p, workspace);
-    case 10: return launch_dma_cfg<64, 64, 32, 32, 64, 4, EPI, TO, WF>(x, w, c, m, n, k, s, p, workspace);
-    case 13: return launch_dma_cfg<128, 64, 32, 64, 128, 3, EPI, TO, WF>(x, w, c, m, n, k, s, p, workspace);
-    case 6: return launch_dma_cfg<192, 256, 96, 64, 64, 2, EPI, TO, WF>(x, w, c, m, n, k, s, p, workspace);
-    case 5: return launch_dma_cfg<128, 128, 64, 64, 64, 2, EPI, TO, WF>(x, w, c, m, n, k, s, p, workspace);
-    case 4: return launch_dma_cfg<256, 256, 128, 64, 64, 2, EPI, TO, WF>(x, w, c, m, n, k, s, p, workspace);
+    case 8: return launch_dma_cfg<256, 128, 64, 64, 64, 3, EPI, TO, WF>(x, w, c, m, n, k, s, p, workspace, act);
+    case 9: return launch_dma_cfg<320, 256, 160, 64, 64, 2, EPI, TO, WF>(x, w, c, m, n, k, s, p, workspace, act);
+    case 7: return launch_dma_cfg<128, 64, 32, 64, 64, 3, EPI, TO, WF>(x, w, c, m, n, k, s, p, workspace, act);
+    case 10: return launch_dma_cfg<64, 64, 32, 32, 64, 4, EPI, TO, WF>(x, w, c, m, n, k, s, p, workspace, act);
+    case 13: return launch_dma_cfg<128, 64, 32, 64, 128, 3, EPI, TO, WF>(x, w, c, m, n, k, s, p, workspace, act);
+    case 6: return launch_dma_cfg<192, 256, 96, 64, 64, 2, EPI, TO, WF>(x, w, c, m, n, k, s, p, workspace, act);
+    case 5: return launch_dma_cfg<128, 128, 64, 64, 64, 2, EPI, TO, WF>(x, w, c, m, n, k, s, p, workspace, act);
+    case 4: return launch_dma_cfg<256, 256, 128, 64, 64, 2, EPI, TO, WF>(x, w, c, m, n, k, s, p, workspace, act);
     default: break;
   }
   if constexpr (!WF) {
     switch (plan.cfg) {
-      case 3: return launch_tiled_cfg<256, 256, 128, 64, 2, EPI, TO>(x, w, c, m, n, k, s);
-      case 2: return launch_tiled_cfg<256, 128, 128, 64, 2, EPI, TO>(x, w, c, m, n, k, s);
-      default: return launch_tiled_cfg<128, 128, 64, 64, 2, EPI, TO>(x, w, c, m, n, k, s);
+      case 3: return launch_tiled_cfg<256, 256, 128, 64, 2, EPI, TO>(x, w, c, m, n, k, s, act);
+      case 2: return launch_tiled_cfg<256, 128, 128, 64, 2, EPI, TO>(x, w, c, m, n, k, s, act);
+      default: return launch_tiled_cfg<128, 128, 64, 64, 2, EPI, TO>(x, w, c, m, n, k, s, act);
     }
   }
   RB_REQUIRE(false, "rb_gemm_bf16: internal: fragment-major W with K=%d, which the direct-to-LDS kernels do not take", k);
@@ -747,7 +762,8 @@ int gemm_tiled_parts(int m, int n, int k, int epilogue) {
 }
 
 int gemm_tiled_launch(const bf16_t* x, const bf16_t* w, bool w_frag, void* c, float* workspace, int dtype_out,
-                      int epilogue, int m, int n, int k, hipStream_t s) {
-  if (w_frag) return RB_BY_OUTPUT(launch_planned, true, x, w, c, workspace, m, n, k, s);
-  return RB_BY_OUTPUT(launch_planned, false, x, w, c, workspace, m, n, k, s);
+                      int epilogue, int m, int n, int k, hipStream_t s, const float* act) {
+  RB_REQUIRE(act == nullptr || epilogue == 0, "rb_gemm_bf16: an activation goes with epilogue 0");
+  if (w_frag) return RB_BY_OUTPUT(launch_planned, true, x, w, c, workspace, m, n, k, s, act);
+  return RB_BY_OUTPUT(launch_planned, false, x, w, c, workspace, m, n, k, s, act);
 }

@@ -133,6 +133,7 @@ class Kernels:
             "rb_swiglu": [_P, _P, _I, _I, _I, _P],
             "rb_gemm_generic": [_P, _P, _I, _P, _I, _I, _I, _I, _I, _P],
             "rb_gemm_bf16": [_P, _P, _I, _P, _I, _I, _I, _I, _I, _P, _P],
+            "rb_gemm_bf16_act": [_P, _P, _I, _P, _I, _I, _P, _I, _I, _I, _P, _P],
             "rb_gemm_bf16_few": [_P, _P, _F, _P, _P, _I, _P, _I, _I, _P, _P, _P, _I, _I, _I, _P],
             "rb_gemm_bf16_few_ok": [_I, _I, _I],
             "rb_gemm_bf16_terms_count": [_I, _I, _I],
@@ -275,8 +276,9 @@ class Kernels:
                                            dtype_code(c.dtype), m, n, k, self._stream()))
 
     def gemm_bf16(self, a: torch.Tensor, w: torch.Tensor, c: torch.Tensor, epilogue: int = 0,
-                  w_frag: bool = False) -> None:
-        """w_frag: w [N, K] is stored fragment-major (`place_rows(..., frag=True)` writes that)."""
+                  w_frag: bool = False, act: Optional[torch.Tensor] = None) -> None:
+        """w_frag: w [N, K] is stored fragment-major (`place_rows(..., frag=True)` writes that).
+        act (epilogue 0): the two numbers of xIELU, float32 [2]; the result is xIELU(a w^T)."""
         m, k = a.shape
         n = w.shape[0]
         _check(a, "a", torch.bfloat16)
@@ -284,8 +286,12 @@ class Kernels:
         _check(c, "c", None, (m, n // 2 if epilogue == 1 else n))
         need = int(self._lib.rb_gemm_workspace_floats(m, n, k, int(epilogue)))
         workspace = torch.empty(need, dtype=torch.float32, device=a.device) if need else None
-        self._ok(self._lib.rb_gemm_bf16(_ptr(a), _ptr(w), int(bool(w_frag)), _ptr(c), dtype_code(c.dtype), int(epilogue),
-                                        m, n, k, _ptr(workspace), self._stream()))
+        if act is not None:
+            _check(act, "act", torch.float32, (2,))
+            if epilogue != 0:
+                raise KernelError("gemm_bf16: an activation goes with epilogue 0")
+        self._ok(self._lib.rb_gemm_bf16_act(_ptr(a), _ptr(w), int(bool(w_frag)), _ptr(c), dtype_code(c.dtype), int(epilogue),
+                                            _ptr(act), m, n, k, _ptr(workspace), self._stream()))
 
     def gemm_bf16_terms_count(self, m: int, n: int, k: int) -> int:
         return int(self._lib.rb_gemm_bf16_terms_count(int(m), int(n), int(k)))

@@ -294,9 +294,6 @@ extern "C" int rb_embed_streams(const void* table, int table_dtype, const int32_
 
 // ---------------------------------------------------------------- xIELU
 // z > 0: softplus(p) z^2 + z / 2;  z <= 0: (1/2 + softplus(q)) (exp(z) - 1 - z) + z / 2, with (p, q) = act[0..1].
-__device__ __forceinline__ float xielu_value(float v, float ap, float an) {
-  return v > 0.f ? fmaf(ap * v, v, 0.5f * v) : fmaf(an, expm1f(v) - v, 0.5f * v);
-}
 __device__ __forceinline__ void xielu_store4(float* p, float a, float b, float c, float d) {
   *reinterpret_cast<float4*>(p) = make_float4(a, b, c, d);
 }
@@ -307,9 +304,8 @@ __device__ __forceinline__ void xielu_store4(bf16_t* p, float a, float b, float 
 // four values a thread with 16-byte loads (n4 quads), then the rest one by one
 template <typename TO>
 __global__ void xielu_kernel(const float* __restrict__ z, const float* __restrict__ act, TO* __restrict__ out, size_t n) {
-  const float p = act[0], q = act[1];
-  const float ap = p > 20.0f ? p : log1pf(expf(p));
-  const float an = 0.5f + (q > 20.0f ? q : log1pf(expf(q)));
+  const XieluPair pair = xielu_pair(act);
+  const float ap = pair.ap, an = pair.an;
   const size_t n4 = n / 4;
   for (size_t e = (size_t)blockIdx.x * blockDim.x + threadIdx.x; e < n4; e += (size_t)gridDim.x * blockDim.x) {
     const float4 v = *reinterpret_cast<const float4*>(z + 4 * e);

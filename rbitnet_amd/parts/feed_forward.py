@@ -18,7 +18,7 @@ import torch
 
 from ..errors import ConfigError
 from .base import BuildEnv, Part, TensorSpec, register_feed_forward
-from .linear import can_fuse_gate, gated_linear, linear, linear_to_stream, pack_gate_up, pack_rows
+from .linear import can_fuse_gate, gated_linear, linear, linear_to_stream, pack_gate_up, pack_rows, xielu_linear
 
 DEFAULT_NAMES = {"gate": "gate_proj.weight", "up": "up_proj.weight", "down": "down_proj.weight"}
 
@@ -86,9 +86,7 @@ class DenseXielu(Part):
 
     def forward(self, h, ctx=None, stream: Optional[torch.Tensor] = None, next_norm=None):
         lib = self.env.lib
-        z = linear(lib, h, self.w_up, torch.float32)
-        t = torch.empty((h.shape[0], self.ff), dtype=self.env.dtype, device=z.device)
-        lib.xielu(z, self.act, t)
+        t = xielu_linear(lib, h, self.w_up, self.act, self.env.dtype)      # the activation in the product's epilogue
         return linear(lib, t, self.w_down, torch.float32)
 
 

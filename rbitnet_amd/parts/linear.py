@@ -133,6 +133,23 @@ def linear_to_stream(lib, x: torch.Tensor, w, stream: Optional[torch.Tensor], ne
     return GainedRows(next_norm, stream, gained, squares)
 
 
+def xielu_linear(lib, x: torch.Tensor, w, act: torch.Tensor, out_dtype: torch.dtype) -> torch.Tensor:
+    """xIELU(x W^T) -> [M, N] in `out_dtype`, act float32 [2] being the activation's two numbers.  On the matrix cores the
+    activation is applied where the product's float32 sums are stored; elsewhere by a kernel of its own on them."""
+    m, k = x.shape
+    n = w.shape[0]
+    out = torch.empty((m, n), dtype=out_dtype, device=x.device)
+    if m == 0:
+        return out
+    wd, frag = _data(w)
+    if uses_matrix_cores(x.dtype, k):
+        lib.gemm_bf16(x, wd, out, 0, w_frag=frag, act=act)
+        return out
+    z = linear(lib, x, w, torch.float32)
+    lib.xielu(z, act, out)
+    return out
+
+
 def can_fuse_gate(dtype: torch.dtype, k: int, ff: int) -> bool:
     """Whether silu(gate) * up can be computed in the product's epilogue."""
     return uses_matrix_cores(dtype, k) and ff % GATE_BLOCK == 0

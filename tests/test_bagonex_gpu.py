@@ -115,6 +115,30 @@ def test_streams_update_xielu_and_cap(lib):
     assert _rel(lg, want) < 2e-6
 
 
+@pytest.mark.parametrize("m,n,k", [(1, 384, 256), (8, 8192, 2048), (16, 16384, 512), (40, 512, 4096), (128, 1024, 8192),
+                                   (300, 2048, 1024), (2048, 4096, 1024), (100, 256, 200), (5, 40, 24), (70, 96, 100)])
+@pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float32])
+def test_xielu_in_the_products_epilogue(lib, m, n, k, out_dtype):
+    """xIELU(x W^T) from the product's own epilogue, for token counts and sizes that reach each of the product kernels
+    (few tokens, rows resident, tiles with and without slices of K, K that is no multiple of 64, sizes off the matrix
+    cores' grid), W stored either way: the float32 sums are activated, then rounded once."""
+    from rbitnet_amd.parts.linear import pack_rows, xielu_linear
+    g = torch.Generator().manual_seed(m + n + k)
+    x = _bf(torch.randn(m, k, generator=g, dtype=F64))
+    w = _bf(torch.randn(n, k, generator=g, dtype=F64) * k ** -0.5 * 2)
+    act = torch.tensor([0.4, -0.3], dtype=F64)
+    want = P.xielu(x @ w.T, act[0], act[1])
+    wd = w.to(DEV, torch.bfloat16)
+    for frag_allowed in (True, False):
+        mat = pack_rows(lib, [(wd, 0, None, None)], n, k, torch.bfloat16, torch.device(DEV), frag_allowed)
+        got = xielu_linear(lib, x.to(DEV, torch.bfloat16), mat, act.float().to(DEV), out_dtype)
+        assert got.dtype == out_dtype and _rel(got, want) < (6e-3 if out_dtype == torch.bfloat16 else 2e-5), frag_allowed
+    if k % 8 == 0:                                   # and the plain product beside it is what it was
+        plain = torch.empty(m, n, dtype=torch.float32, device=DEV)
+        lib.gemm_bf16(x.to(DEV, torch.bfloat16), wd, plain, 0)
+        assert _rel(plain, x @ w.T) < 2e-5
+
+
 @pytest.mark.parametrize("taps", [1, 2, 4])
 @pytest.mark.parametrize("residual,act", [(True, ACT_NONE), (False, ACT_SILU)])
 def test_short_convolution_in_pieces_and_batches(lib, taps, residual, act):
