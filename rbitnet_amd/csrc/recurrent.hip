@@ -15,31 +15,61 @@ __device__ __forceinline__ float rb_softplus(float v) { return v > 20.0f ? v : l
 // y[t, c] = (residual ? x[t, c] : 0) + sum_d w[c, taps - 1 - d] * x[t - d, c], d = 0 .. taps - 1, where rows
 // before the step's first come from the sequence's state (its last taps - 1 inputs, oldest first) and rows
 // before the sequence's start are zero (the state of a fresh slot is zero).  act 1: silu on the result.
-// Afterwards the state holds the last taps - 1 inputs again.  One launch: a workgroup per token for the tokens
-// that need rows of the step only, and a workgroup per sequence that walks the step's first taps - 1 tokens with
+// Afterwards the state holds the last taps - 1 inputs again.  One launch: workgroups that walk 16 rows each of the
+// tokens that need rows of the step only, and a workgroup per sequence that walks the step's first taps - 1 tokens with
 // the old state in registers and then writes the new state, so that whoever reads the state is also who writes it.
 #define SC_MAX_TAPS 16
+#define SC_TILE 16             // rows of the step that a workgroup walks
 template <typename TO>
 __global__ void short_conv_kernel(const float* __restrict__ x, size_t x_stride, const float* __restrict__ w, int taps,
                                   float* __restrict__ state, const int32_t* __restrict__ tok_pos,
                                   const int32_t* __restrict__ tok_seq, const int32_t* __restrict__ cu_seqlens,
                                   const int32_t* __restrict__ slots, TO* __restrict__ out, size_t out_stride,
-                                  int residual, int act, int channels, int n_tokens) {
+                                  int residual, int act, int channels, int n_tokens, int n_tiles) {
   const int keep = taps - 1;
-  if ((int)blockIdx.x < n_tokens) {
-    const int t = blockIdx.x;
-    if (t - cu_seqlens[tok_seq[t]] < keep) return;           // the sequence's workgroup takes it
+  if ((int)blockIdx.x < n_tiles) {
+    // SC_TILE rows of the packed step, walked with the window (the last taps - 1 inputs) in registers: one new row a
+    // token.  Rows that are among a sequence's first taps - 1 of the step belong to the sequence's workgroup; after such
+    // a row (and at the tile's start) the window is read anew.
+    const int r0 = blockIdx.x * SC_TILE;
+    const int r1 = r0 + SC_TILE < n_tokens ? r0 + SC_TILE : n_tokens;
     for (int c = blockIdx.y * blockDim.x + threadIdx.x; c < channels; c += gridDim.y * blockDim.x) {
-      const float cur = x[(size_t)t * x_stride + c];
-      float acc = residual ? cur : 0.f;
-      for (int d = 0; d < taps; ++d)
-        acc = fmaf(w[(size_t)c * taps + (keep - d)], d == 0 ? cur : x[(size_t)(t - d) * x_stride + c], acc);
-      if (act == 1) acc = acc * rb_sigmoid(acc);
-      Num<TO>::store(out + (size_t)t * out_stride + c, acc);
+      float win[SC_MAX_TAPS], wt[SC_MAX_TAPS];
+#pragma unroll
+      for (int j = 0; j < SC_MAX_TAPS; ++j) {
+        win[j] = 0.f;
+        wt[j] = j < keep ? w[(size_t)c * taps + j] : 0.f;
+      }
+      const float w_cur = w[(size_t)c * taps + keep];
+      bool have = false;
+      for (int t = r0; t < r1; ++t) {
+        if (t - cu_seqlens[tok_seq[t]] < keep) {             // the sequence's workgroup takes it
+          have = false;
+          continue;
+        }
+        if (!have) {
+#pragma unroll
+          for (int j = 0; j < SC_MAX_TAPS; ++j)
+            if (j < keep) win[j] = x[(size_t)(t - keep + j) * x_stride + c];
+          have = true;
+        }
+        const float cur = x[(size_t)t * x_stride + c];
+        float acc = residual ? cur : 0.f;
+        acc = fmaf(w_cur, cur, acc);
+#pragma unroll
+        for (int j = 0; j < SC_MAX_TAPS; ++j) acc = fmaf(wt[j], win[j], acc);
+#pragma unroll
+        for (int j = 0; j < SC_MAX_TAPS - 1; ++j) win[j] = j + 1 < keep ? win[j + 1] : win[j];
+#pragma unroll
+        for (int j = 0; j < SC_MAX_TAPS; ++j)
+          if (j == keep - 1) win[j] = cur;
+        if (act == 1) acc = acc * rb_sigmoid(acc);
+        Num<TO>::store(out + (size_t)t * out_stride + c, acc);
+      }
     }
     return;
   }
-  const int b = blockIdx.x - n_tokens;
+  const int b = blockIdx.x - n_tiles;
   const int row0 = cu_seqlens[b], n = cu_seqlens[b + 1] - row0;
   float* st = state + (size_t)slots[b] * keep * channels;
   const int first = n < keep ? n : keep;
@@ -86,14 +116,15 @@ extern "C" int rb_short_conv(const float* x, long long x_stride, const float* w,
   RB_REQUIRE(taps == 1 || state != nullptr, "rb_short_conv: %d taps need a state", taps);
   RB_REQUIRE(act == 0 || act == 1, "rb_short_conv: unknown activation %d", act);
   if (n_tokens == 0) return 0;
-  dim3 grid(n_tokens + (taps > 1 ? n_seqs : 0), (channels + 255) / 256 < 16 ? (channels + 255) / 256 : 16);
+  const int n_tiles = (n_tokens + SC_TILE - 1) / SC_TILE;
+  dim3 grid(n_tiles + (taps > 1 ? n_seqs : 0), (channels + 255) / 256 < 64 ? (channels + 255) / 256 : 64);
   hipStream_t s = (hipStream_t)stream;
   if (out_dtype == RB_F32)
     short_conv_kernel<float><<<grid, 256, 0, s>>>(x, (size_t)x_stride, w, taps, state, tok_pos, tok_seq, cu_seqlens, slots,
-                                                  (float*)out, (size_t)out_stride, residual, act, channels, n_tokens);
+                                                  (float*)out, (size_t)out_stride, residual, act, channels, n_tokens, n_tiles);
   else if (out_dtype == RB_BF16)
     short_conv_kernel<bf16_t><<<grid, 256, 0, s>>>(x, (size_t)x_stride, w, taps, state, tok_pos, tok_seq, cu_seqlens, slots,
-                                                   (bf16_t*)out, (size_t)out_stride, residual, act, channels, n_tokens);
+                                                   (bf16_t*)out, (size_t)out_stride, residual, act, channels, n_tokens, n_tiles);
   else
     RB_REQUIRE(false, "rb_short_conv: unknown dtype %d", out_dtype);
   RB_LAUNCH_CHECK();
