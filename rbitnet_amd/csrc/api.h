@@ -93,7 +93,7 @@ int rb_gemm_bf16_few(const void* a, const float* squares_in, float eps, const in
                      float* squares_out, int m, int n, int k, void* stream);
 
 // Causal attention of every token over its sequence's cache (keys 0..pos, or the last
-// `window` of them), any head_dim that is even and at most 512.
+// `window` of them), any head_dim up to 512 (a rotation in front of it needs an even one).
 //   q [T, Hq, D], out [T, Hq * D], both of dtype; pages as in rb_rope_kv_write.
 int rb_attention_generic(const void* q, const void* k_pages, const void* v_pages, void* out, int dtype,
                          const int32_t* tok_pos, const int32_t* tok_seq, const int32_t* block_table,

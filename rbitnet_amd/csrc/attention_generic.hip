@@ -1,4 +1,4 @@
-// Causal attention of each token over its sequence's paged cache: any even head_dim up to
+// Causal attention of each token over its sequence's paged cache: any head_dim up to
 // 512, any number of heads and groups, float32 or bfloat16 storage, float32 arithmetic
 // throughout (scores, softmax, weighted sum).  One workgroup per (token, query head): one wave
 // when the step has many tokens, up to 8 waves that share the pages of the context and merge
@@ -278,8 +278,8 @@ extern "C" int rb_attention_generic_sinks(const void* q, const void* k_pages, co
                                          n_heads, n_kv_heads, head_dim, scale, window, sinks, stream));
   RB_REQUIRE(n_tokens >= 0 && n_heads > 0 && n_kv_heads > 0 && n_heads % n_kv_heads == 0,
              "rb_attention_generic: bad head counts Hq=%d Hk=%d", n_heads, n_kv_heads);
-  RB_REQUIRE(head_dim > 0 && head_dim % 2 == 0 && head_dim <= AG_MAX_D,
-             "rb_attention_generic: head_dim %d not supported (even, at most %d)", head_dim, AG_MAX_D);
+  RB_REQUIRE(head_dim > 0 && head_dim <= AG_MAX_D, "rb_attention_generic: head_dim %d not supported (at most %d)", head_dim,
+             AG_MAX_D);
   RB_REQUIRE(n_heads <= 65535, "rb_attention_generic: too many heads %d", n_heads);
   RB_REQUIRE(window >= 0, "rb_attention_generic: negative window");
   if (n_tokens == 0) return 0;

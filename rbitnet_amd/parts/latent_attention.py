@@ -45,8 +45,8 @@ class LatentAttention(Part):
         self.eps = float(params["eps"])
         self.cache_from = params.get("cache_from")
         self.window = None
-        if self.kv_rank <= 0 or self.kv_rank % 2 != 0 or self.kv_rank > MAX_RANK:
-            raise ConfigError(f"latent attention: kv_rank {self.kv_rank} not supported (even, at most {MAX_RANK})")
+        if self.kv_rank <= 0 or self.kv_rank > MAX_RANK:
+            raise ConfigError(f"latent attention: kv_rank {self.kv_rank} not supported (at most {MAX_RANK})")
         if min(self.heads, self.dim, self.vdim, self.q_rank) <= 0:
             raise ConfigError("latent attention: sizes must be positive")
         if self.dim > 768:

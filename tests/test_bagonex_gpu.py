@@ -270,7 +270,7 @@ def _latent_weights(hidden, h, dk, dv, qr, kr, seed):
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("h,dk,dv,qr,kr,scale", [(4, 16, 24, 40, 32, 0.25), (1, 64, 8, 16, 64, 0.1), (5, 8, 8, 24, 18, 0.6),
-                                                 (2, 32, 32, 32, 128, 0.2), (3, 16, 8, 24, 320, 0.1)])
+                                                 (2, 32, 32, 32, 128, 0.2), (3, 16, 8, 24, 320, 0.1), (2, 7, 5, 9, 33, 0.4)])
 def test_latent_attention_whole_in_pieces_and_token_by_token(lib, dtype, h, dk, dv, qr, kr, scale):
     hidden, t_len = 48, 150
     params = {"heads": h, "dim": dk, "vdim": dv, "q_rank": qr, "kv_rank": kr, "scale": scale, "eps": 1e-5, "cache_from": None}
