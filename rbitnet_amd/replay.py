@@ -136,8 +136,8 @@ def main(argv: Optional[list] = None) -> int:
         from .cache import PAGE_SIZE
         from .engine import Engine
         # every live request holds at least one token and may leave most of its last page empty: room for that
-        # many requests (64 at most), and a page more for each than their tokens alone would take
-        slots = max(1, min(int(args.max_tokens), 64))
+        # many requests (256 at most), and a page more for each than their tokens alone would take
+        slots = max(1, min(int(args.max_tokens), 256))
         engine = Engine.load_path(args.model, dtype=args.dtype, max_tokens=int(args.max_tokens) + PAGE_SIZE * slots,
                                   max_batch=slots)
         replay(engine, sys.stdin, args.out)
