@@ -19,6 +19,7 @@ from typing import Any, Dict, Iterable, Optional, Tuple
 from ..errors import ConfigError
 from .bagonex import BagonexConfig
 from .llama import LlamaConfig
+from .tigutar import TigutarConfig
 from .spec import ModelSpec
 
 _ARCHITECTURES: Dict[str, Any] = {}
@@ -95,3 +96,4 @@ def load_config(path_or_dict: Any, tensor_names: Optional[Iterable[str]] = None,
 
 register_architecture("LlamaForCausalLM", LlamaConfig)
 register_architecture("Bagonex", BagonexConfig)
+register_architecture("Tigutar", TigutarConfig)

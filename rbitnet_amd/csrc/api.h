@@ -187,6 +187,58 @@ int rb_delta_rule(const float* q, const float* k, long long qk_stride, const flo
 int rb_gated_rmsnorm(const float* o, const float* weight, const float* gate, long long gate_stride, float eps, void* out,
                      int out_dtype, int n_tokens, int n_heads, int vdim, void* stream);
 
+// rb_delta_prep with its choices spelled out.  unit 1: q and k heads become unit vectors (q times q_scale); 0: q is
+// only multiplied by q_scale.  The a_cols numbers of a row of `a` (a_cols = H: one decay per head; H * dim: one per head
+// and key channel) become decays in place: decay 0: exp(-exp(a_log[head]) softplus(a + bias[i])); decay 1:
+// sigmoid(a + bias[i]) ^ (1 / tau).  bias may be null.  b_in null: no beta.
+int rb_recurrence_prep(float* qk, long long qk_stride, int n_kv_heads, int dim, int unit, float q_scale, float unit_eps, float* a,
+                       long long a_stride, int a_cols, int decay, const float* bias, const float* a_log, float tau, int n_heads,
+                       const float* b_in, long long b_stride, float* beta, int n_tokens, void* stream);
+// rb_delta_rule with one decay per head (g_per_head 1: g[t * g_stride + h]) or per key channel (0), and, with beta null,
+// the plain rule without the correction:  S <- diag(g) S + k v^T;  out = S^T q.
+int rb_linear_recurrence(const float* q, const float* k, long long qk_stride, const float* v, long long v_stride, const float* g,
+                         long long g_stride, int g_per_head, const float* beta, float* state, const int32_t* cu_seqlens,
+                         const int32_t* slots, float* out, int n_seqs, int n_tokens, int n_heads, int n_kv_heads, int dim, int vdim,
+                         void* stream);
+// rb_gated_rmsnorm with the gate's activation: act 0 sigmoid(gate), 1 silu(gate).
+int rb_gated_rmsnorm_act(const float* o, const float* weight, const float* gate, long long gate_stride, int act, float eps, void* out,
+                         int out_dtype, int n_tokens, int n_heads, int vdim, void* stream);
+
+// ---- a plain stream with layer norm (streams.hip)
+// v = x[src] + dscale * (delta[src] + (delta2 ? delta2[src] : 0)), src = rows ? rows[r] : r; without rows x[src] = v too;
+// out[r] = (v - mean) / sqrt(var + eps) * weight + bias.  delta null: the norm alone.
+int rb_layernorm_residual(float* x, const float* delta, const float* delta2, float dscale, const float* weight, const float* bias,
+                          float eps, const int32_t* rows, int n_rows, int width, void* out, int out_dtype, void* stream);
+
+// ---- around the mixers (mixers.hip)
+// rb_rope_kv_write for heads whose keys and values differ in size and of which only the first `rot` numbers are rotated
+// (i paired with i + rot / 2; cos, sin [positions, rot / 2]).  A row of qkv (row_width floats apart) holds Hq and Hk
+// heads of `dim` and Hk heads of `vdim`; q_out [T, Hq, pad] and the pages [*, Hk, 64, pad] get them padded with zeros.
+int rb_rope_store(const float* qkv, long long row_width, const float* cos, const float* sin, int rot, void* q_out, void* k_pages,
+                  void* v_pages, int cache_dtype, const int32_t* tok_pos, const int32_t* tok_seq, const int32_t* block_table,
+                  int bt_stride, int n_tokens, int n_heads, int n_kv_heads, int dim, int vdim, int pad, void* stream);
+// x[t, h, :] *= sigmoid(gate[t * gate_stride + h]); x [T, H, D] of dtype, in place.
+int rb_head_gate(void* x, int dtype, const float* gate, long long gate_stride, int n_tokens, int n_heads, int head_dim, void* stream);
+// out = (rmsnorm(a) * wa + rmsnorm(b) * wb) / 2 over rows of `width` float32 numbers.
+int rb_pair_norm_mean(const float* a, const float* wa, const float* b, const float* wb, float eps, float* out, int n_tokens,
+                      int width, void* stream);
+
+// ---- a feed-forward of routed experts (routed.hip)
+// Router logits z [T, z_stride >= experts] -> the `top` experts with the largest sigmoid(z) per token (lowest index among
+// equals): sel, weight [T * top] (pair p = t * top + k), and the pairs sorted by expert in runs padded to 16 rows:
+// row_pair [max_rows] (-1: padding), tile_expert [max_rows / 16] (-1: past the end).  max_rows: a multiple of 16, at
+// least T * top rounded up to 16, plus 16 for every expert.
+int rb_route_top(const float* z, long long z_stride, int n_experts, int top, int32_t* sel, float* weight, int32_t* row_pair,
+                 int32_t* tile_expert, int max_rows, int n_tokens, void* stream);
+// For every pair p of token t: x = weight[p] h[t]; g = min(Wg x, limit), u = clamp(Wu x, -limit, limit);
+// out[p] = Wd (g sigmoid(alpha g) (u + 1)), the expert being the pair's.  w_gate, w_up [experts, ff, width] and w_down
+// [experts, width, ff] of dtype; y [max_rows, ff] of dtype is scratch; out [T * top, width] float32.
+int rb_routed_experts(const void* h, int dtype, const float* weight, int top, const int32_t* row_pair, const int32_t* tile_expert,
+                      int max_rows, const void* w_gate, const void* w_up, const void* w_down, void* y, float* out, int n_experts,
+                      int width, int ff, float limit, float alpha, void* stream);
+// out[t] = sum over k of pairs[t * top + k], in the order of k.
+int rb_pairs_sum(const float* pairs, int top, float* out, int n_tokens, int width, void* stream);
+
 // ---- attention through a latent (latent.hip)
 // Per token: cq = rmsnorm(proj[t, 0:q_rank]) * q_gain -> cq [T, q_rank]; rmsnorm(proj[t, kv_col:+kv_rank]) * kv_gain ->
 // the token's place in pages [n_pages, 1, 64, kv_rank].  A rank of 0 leaves that half out.

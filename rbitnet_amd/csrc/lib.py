@@ -105,7 +105,8 @@ class KernelTimes:
         return "\n".join(lines)
 
 
-TIMED_OPS = ("embed_streams", "streams_layernorm", "streams_update", "xielu", "tanh_cap", "short_conv",
+TIMED_OPS = ("recurrence_prep", "linear_recurrence", "layernorm_residual", "rope_store", "head_gate", "pair_norm_mean",
+             "route_top", "routed_experts", "pairs_sum", "embed_streams", "streams_layernorm", "streams_update", "xielu", "tanh_cap", "short_conv",
              "delta_prep", "delta_rule", "gated_rmsnorm", "latent_norm_store", "heads_linear", "attention_sinks", "embed_gather", "add_rmsnorm", "rope_kv_write", "swiglu", "gemm_generic", "gemm_bf16", "gemm_bf16_terms",
              "gemm_bf16_few", "attention_generic", "attention_prefill_bf16", "attention_decode_bf16",
              "attention_decode_fused_bf16", "sample")
@@ -163,6 +164,16 @@ class Kernels:
             "rb_gated_rmsnorm": [_P, _P, _P, _L, _F, _P, _I, _I, _I, _I, _P],
             "rb_latent_norm_store": [_P, _L, _I, _P, _P, _I, _I, _P, _P, _I, _P, _P, _P, _I, _F, _I, _P],
             "rb_heads_linear": [_P, _I, _P, _I, _P, _I, _I, _I, _I, _I, _P],
+            "rb_recurrence_prep": [_P, _L, _I, _I, _I, _F, _F, _P, _L, _I, _I, _P, _P, _F, _I, _P, _L, _P, _I, _P],
+            "rb_linear_recurrence": [_P, _P, _L, _P, _L, _P, _L, _I, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P],
+            "rb_gated_rmsnorm_act": [_P, _P, _P, _L, _I, _F, _P, _I, _I, _I, _I, _P],
+            "rb_layernorm_residual": [_P, _P, _P, _F, _P, _P, _F, _P, _I, _I, _P, _I, _P],
+            "rb_rope_store": [_P, _L, _P, _P, _I, _P, _P, _P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P],
+            "rb_head_gate": [_P, _I, _P, _L, _I, _I, _I, _P],
+            "rb_pair_norm_mean": [_P, _P, _P, _P, _F, _P, _I, _I, _P],
+            "rb_route_top": [_P, _L, _I, _I, _P, _P, _P, _P, _I, _I, _P],
+            "rb_routed_experts": [_P, _I, _P, _I, _P, _P, _I, _P, _P, _P, _P, _P, _I, _I, _I, _F, _F, _P],
+            "rb_pairs_sum": [_P, _I, _P, _I, _I, _P],
         }
         for name, args in sig.items():
             fn = getattr(L, name)
@@ -588,6 +599,195 @@ class Kernels:
         _check(out, "out", None, (n, n_heads * vdim))
         self._ok(self._lib.rb_gated_rmsnorm(_ptr(o), _ptr(weight), gate.data_ptr() + 4 * gate_col, gate.shape[1], float(eps),
                                             _ptr(out), dtype_code(out.dtype), n, n_heads, vdim, self._stream()))
+
+    # ------------------------------------------------------------------ recurrences with their choices spelled out
+    def recurrence_prep(self, qkv: torch.Tensor, n_kv: int, dim: int, unit: bool, q_scale: float, unit_eps: float,
+                        a: torch.Tensor, a_col: int, a_cols: int, decay: int, bias: Optional[torch.Tensor],
+                        a_log: Optional[torch.Tensor], tau: float, n_heads: int, b_in: Optional[torch.Tensor] = None,
+                        b_col: int = 0, beta: Optional[torch.Tensor] = None) -> None:
+        """In place: the q and k heads at the start of qkv's rows (unit vectors, or q only scaled), and columns
+        a_col .. a_col + a_cols of `a` turned into decays (a_cols = heads: one per head; heads * dim: per key channel;
+        decay 0: exp(-exp(a_log) softplus(a + bias)), 1: sigmoid(a + bias) ^ (1 / tau)); beta [T, H] from b_in's columns."""
+        n, width = qkv.shape
+        _check(qkv, "qkv", torch.float32)
+        if width < 2 * n_kv * dim:
+            raise KernelError("recurrence_prep: rows too short for the q and k heads")
+        _check(a, "a", torch.float32)
+        if a.shape[0] != n or a_col < 0 or a_col + a_cols > a.shape[1] or a_cols not in (n_heads, n_heads * dim):
+            raise KernelError("recurrence_prep: the decays' columns lie outside the rows, or are not one per head or channel")
+        if bias is not None:
+            _check(bias, "bias", torch.float32, (a_cols,))
+        if decay == 0:
+            _check(a_log, "a_log", torch.float32, (n_heads,))
+        b_ptr, b_stride = None, 0
+        if b_in is not None:
+            _check(b_in, "b_in", torch.float32)
+            if b_in.shape[0] != n or b_col < 0 or b_col + n_heads > b_in.shape[1]:
+                raise KernelError("recurrence_prep: the beta columns lie outside the rows")
+            _check(beta, "beta", torch.float32, (n, n_heads))
+            b_ptr, b_stride = b_in.data_ptr() + 4 * b_col, b_in.shape[1]
+        self._ok(self._lib.rb_recurrence_prep(_ptr(qkv), width, n_kv, dim, int(bool(unit)), float(q_scale), float(unit_eps),
+                                              a.data_ptr() + 4 * a_col, a.shape[1], a_cols, int(decay), _ptr(bias), _ptr(a_log),
+                                              float(tau), n_heads, b_ptr, b_stride, _ptr(beta), n, self._stream()))
+
+    def linear_recurrence(self, qkv: torch.Tensor, n_kv: int, dim: int, n_heads: int, vdim: int, g: torch.Tensor, g_col: int,
+                          g_per_head: bool, beta: Optional[torch.Tensor], state: torch.Tensor, ctx, out: torch.Tensor) -> None:
+        """`delta_rule` with the decays at columns g_col .. of g, one per head (g_per_head) or per head and key channel,
+        and, without beta, the plain rule S <- diag(g) S + k v^T."""
+        n, width = qkv.shape
+        _check(qkv, "qkv", torch.float32)
+        if width < 2 * n_kv * dim + n_heads * vdim:
+            raise KernelError("linear_recurrence: rows too short for q, k and v")
+        _check(g, "g", torch.float32)
+        if g.shape[0] != n or g_col < 0 or g_col + n_heads * (1 if g_per_head else dim) > g.shape[1]:
+            raise KernelError("linear_recurrence: the decays' columns lie outside the rows")
+        if beta is not None:
+            _check(beta, "beta", torch.float32, (n, n_heads))
+        _check(state, "state", torch.float32)
+        if tuple(state.shape[1:]) != (n_heads, vdim, dim):
+            raise KernelError(f"linear_recurrence: state of shape {tuple(state.shape)}, expected [*, {n_heads}, {vdim}, {dim}]")
+        _check(out, "out", torch.float32, (n, n_heads * vdim))
+        if ctx.n_tokens != n:
+            raise KernelError("linear_recurrence: the step's tokens and the rows differ")
+        base = qkv.data_ptr()
+        self._ok(self._lib.rb_linear_recurrence(base, base + 4 * n_kv * dim, width, base + 8 * n_kv * dim, width,
+                                                g.data_ptr() + 4 * g_col, g.shape[1], int(bool(g_per_head)), _ptr(beta), _ptr(state),
+                                                _ptr(ctx.cu_seqlens), _ptr(ctx.slots), _ptr(out), ctx.n_seqs, n, n_heads, n_kv, dim,
+                                                vdim, self._stream()))
+
+    def gated_rmsnorm_act(self, o: torch.Tensor, weight: torch.Tensor, gate: torch.Tensor, gate_col: int, act: int, eps: float,
+                          n_heads: int, vdim: int, out: torch.Tensor) -> None:
+        """`gated_rmsnorm` with the gate's activation: 0 sigmoid, 1 silu."""
+        n = o.shape[0]
+        _check(o, "o", torch.float32, (n, n_heads * vdim))
+        _check(weight, "weight", torch.float32, (vdim,))
+        _check(gate, "gate", torch.float32)
+        if gate.shape[0] != n or gate_col < 0 or gate_col + n_heads * vdim > gate.shape[1]:
+            raise KernelError("gated_rmsnorm: the gate's columns lie outside the rows")
+        _check(out, "out", None, (n, n_heads * vdim))
+        self._ok(self._lib.rb_gated_rmsnorm_act(_ptr(o), _ptr(weight), gate.data_ptr() + 4 * gate_col, gate.shape[1], int(act),
+                                                float(eps), _ptr(out), dtype_code(out.dtype), n, n_heads, vdim, self._stream()))
+
+    def layernorm_residual(self, x: torch.Tensor, delta: Optional[torch.Tensor], delta2: Optional[torch.Tensor], dscale: float,
+                           weight: torch.Tensor, bias: Optional[torch.Tensor], eps: float, rows: Optional[torch.Tensor],
+                           out: torch.Tensor) -> None:
+        """Layer norm of x [T, E] + dscale * (delta + delta2); without rows the sum is written back to x."""
+        n, width = x.shape
+        _check(x, "x", torch.float32)
+        for name, d in (("delta", delta), ("delta2", delta2)):
+            if d is not None:
+                _check(d, name, torch.float32, (n, width))
+        if delta is None and delta2 is not None:
+            raise KernelError("layernorm_residual: a second term without a first")
+        _check(weight, "weight", torch.float32, (width,))
+        if bias is not None:
+            _check(bias, "bias", torch.float32, (width,))
+        n_rows = n
+        if rows is not None:
+            n_rows = rows.shape[0]
+            _check(rows, "rows", torch.int32, (n_rows,))
+        _check(out, "out", None, (n_rows, width))
+        self._ok(self._lib.rb_layernorm_residual(_ptr(x), _ptr(delta), _ptr(delta2), float(dscale), _ptr(weight), _ptr(bias),
+                                                 float(eps), _ptr(rows), n_rows, width, _ptr(out), dtype_code(out.dtype),
+                                                 self._stream()))
+
+    # ------------------------------------------------------------------ around the mixers
+    def rope_store(self, qkv: torch.Tensor, cos, sin, rot: int, q_out: torch.Tensor, k_pages, v_pages, tok_pos, tok_seq,
+                   block_table, n_heads: int, n_kv: int, dim: int, vdim: int, pad: int) -> None:
+        """qkv [T, Hq dim (+ Hk dim + Hk vdim)] float32 -> q_out [T, Hq, pad] and the pages [*, Hk, 64, pad], the first
+        `rot` numbers of every q and k head rotated (i with i + rot / 2), heads padded with zeros."""
+        n, width = qkv.shape
+        _check(qkv, "qkv", torch.float32)
+        _check(q_out, "q_out", None, (n, n_heads, pad))
+        _check(tok_pos, "tok_pos", torch.int32, (n,))
+        _check(tok_seq, "tok_seq", torch.int32, (n,))
+        if rot:
+            _check(cos, "cos", torch.float32)
+            _check(sin, "sin", torch.float32, cos.shape)
+            if cos.shape[1] != rot // 2:
+                raise KernelError("angle table width mismatch")
+        need = n_heads * dim
+        if k_pages is not None:
+            need += n_kv * (dim + vdim)
+            _check(block_table, "block_table", torch.int32)
+            _check(k_pages, "k_pages", q_out.dtype)
+            _check(v_pages, "v_pages", q_out.dtype, k_pages.shape)
+            if tuple(k_pages.shape[1:]) != (n_kv, self.page_size, pad):
+                raise KernelError(f"cache pages have shape {tuple(k_pages.shape)}, expected [*, {n_kv}, {self.page_size}, {pad}]")
+        if width < need:
+            raise KernelError("rope_store: rows too short for the heads")
+        self._ok(self._lib.rb_rope_store(_ptr(qkv), width, _ptr(cos), _ptr(sin), int(rot), _ptr(q_out), _ptr(k_pages), _ptr(v_pages),
+                                         dtype_code(q_out.dtype), _ptr(tok_pos), _ptr(tok_seq),
+                                         _ptr(block_table) if k_pages is not None else None,
+                                         block_table.shape[1] if k_pages is not None else 0, n, n_heads, n_kv if k_pages is not None else 0,
+                                         dim, vdim, pad, self._stream()))
+
+    def head_gate(self, x: torch.Tensor, gate: torch.Tensor, gate_col: int, n_heads: int, head_dim: int) -> None:
+        """x [T, H * D] *= sigmoid(gate[:, gate_col + h]) per head, in place."""
+        n = x.shape[0]
+        _check(x, "x", None, (n, n_heads * head_dim))
+        _check(gate, "gate", torch.float32)
+        if gate.shape[0] != n or gate_col < 0 or gate_col + n_heads > gate.shape[1]:
+            raise KernelError("head_gate: the gate's columns lie outside the rows")
+        self._ok(self._lib.rb_head_gate(_ptr(x), dtype_code(x.dtype), gate.data_ptr() + 4 * gate_col, gate.shape[1], n, n_heads,
+                                        head_dim, self._stream()))
+
+    def pair_norm_mean(self, a: torch.Tensor, wa: torch.Tensor, b: torch.Tensor, wb: torch.Tensor, eps: float,
+                       out: torch.Tensor) -> None:
+        n, width = a.shape
+        _check(a, "a", torch.float32)
+        _check(b, "b", torch.float32, (n, width))
+        _check(wa, "wa", torch.float32, (width,))
+        _check(wb, "wb", torch.float32, (width,))
+        _check(out, "out", torch.float32, (n, width))
+        self._ok(self._lib.rb_pair_norm_mean(_ptr(a), _ptr(wa), _ptr(b), _ptr(wb), float(eps), _ptr(out), n, width, self._stream()))
+
+    # ------------------------------------------------------------------ routed experts
+    @staticmethod
+    def routed_rows(n_tokens: int, top: int, n_experts: int) -> int:
+        """Rows that the sorted pairs of a step may take: every expert's run is padded to 16."""
+        return (n_tokens * top + 15) // 16 * 16 + 16 * n_experts
+
+    def route_top(self, z: torch.Tensor, n_experts: int, top: int, sel: torch.Tensor, weight: torch.Tensor,
+                  row_pair: torch.Tensor, tile_expert: torch.Tensor) -> None:
+        n = z.shape[0]
+        _check(z, "z", torch.float32)
+        if z.shape[1] < n_experts:
+            raise KernelError("route_top: rows too short for the experts")
+        max_rows = row_pair.shape[0]
+        if max_rows < self.routed_rows(n, top, n_experts) or max_rows % 16:
+            raise KernelError("route_top: too little room for the sorted pairs")
+        _check(sel, "sel", torch.int32, (n * top,))
+        _check(weight, "weight", torch.float32, (n * top,))
+        _check(row_pair, "row_pair", torch.int32, (max_rows,))
+        _check(tile_expert, "tile_expert", torch.int32, (max_rows // 16,))
+        self._ok(self._lib.rb_route_top(_ptr(z), z.shape[1], n_experts, top, _ptr(sel), _ptr(weight), _ptr(row_pair),
+                                        _ptr(tile_expert), max_rows, n, self._stream()))
+
+    def routed_experts(self, h: torch.Tensor, weight: torch.Tensor, top: int, row_pair: torch.Tensor, tile_expert: torch.Tensor,
+                       w_gate: torch.Tensor, w_up: torch.Tensor, w_down: torch.Tensor, y: torch.Tensor, out: torch.Tensor,
+                       limit: float, alpha: float) -> None:
+        n, width = h.shape
+        n_experts, ff, _ = w_gate.shape
+        max_rows = row_pair.shape[0]
+        _check(h, "h")
+        _check(weight, "weight", torch.float32, (n * top,))
+        _check(row_pair, "row_pair", torch.int32)
+        _check(tile_expert, "tile_expert", torch.int32, (max_rows // 16,))
+        _check(w_gate, "w_gate", h.dtype, (n_experts, ff, width))
+        _check(w_up, "w_up", h.dtype, (n_experts, ff, width))
+        _check(w_down, "w_down", h.dtype, (n_experts, width, ff))
+        _check(y, "y", h.dtype, (max_rows, ff))
+        _check(out, "out", torch.float32, (n * top, width))
+        self._ok(self._lib.rb_routed_experts(_ptr(h), dtype_code(h.dtype), _ptr(weight), top, _ptr(row_pair), _ptr(tile_expert),
+                                             max_rows, _ptr(w_gate), _ptr(w_up), _ptr(w_down), _ptr(y), _ptr(out), n_experts, width,
+                                             ff, float(limit), float(alpha), self._stream()))
+
+    def pairs_sum(self, pairs: torch.Tensor, top: int, out: torch.Tensor) -> None:
+        n, width = out.shape
+        _check(pairs, "pairs", torch.float32, (n * top, width))
+        _check(out, "out", torch.float32)
+        self._ok(self._lib.rb_pairs_sum(_ptr(pairs), top, _ptr(out), n, width, self._stream()))
 
     # ------------------------------------------------------------------ attention through a latent
     def latent_norm_store(self, proj: torch.Tensor, q_rank: int, q_gain: Optional[torch.Tensor], cq: Optional[torch.Tensor],

@@ -131,48 +131,78 @@ extern "C" int rb_short_conv(const float* x, long long x_stride, const float* w,
   return 0;
 }
 
-// ---------------------------------------------------------------- gated delta rule: what enters the recurrence
-// Per token, in place: every q and k head becomes a unit vector, x / sqrt(sum x^2 + unit_eps), q times q_scale;
-// a[t, h, i] becomes the decay exp(-exp(a_log[h]) * softplus(a + dt_bias[h, i])); beta[t, h] = sigmoid(b[t, h]).
-__global__ __launch_bounds__(1024) void delta_prep_kernel(float* __restrict__ qk, size_t qk_stride, int n_kv, int dim, float* __restrict__ a,
-                                  size_t a_stride, const float* __restrict__ dt_bias, const float* __restrict__ a_log, int n_heads,
+// ---------------------------------------------------------------- what enters a recurrence
+// Per token, in place.  The q and k heads (n_kv of each, `dim` numbers): unit 1 makes each a unit vector,
+// x / sqrt(sum x^2 + unit_eps); q is also multiplied by q_scale (unit 0: only that).  The a_cols numbers of a row of
+// `a` become decays, a_cols being H (one per head) or H * dim (one per head and key channel), h = i / (a_cols / H):
+//   decay 0:  exp(-exp(a_log[h]) * softplus(a + bias[i]))
+//   decay 1:  sigmoid(a + bias[i]) ^ (1 / tau), computed as exp(-softplus(-(a + bias[i])) / tau)
+// beta[t, h] = sigmoid(b[t, h]) where b_in is given.
+__global__ __launch_bounds__(1024) void recurrence_prep_kernel(float* __restrict__ qk, size_t qk_stride, int n_kv, int dim, int unit,
+                                  float* __restrict__ a, size_t a_stride, int a_cols, int decay, const float* __restrict__ bias,
+                                  const float* __restrict__ a_log, float tau, int n_heads,
                                   const float* __restrict__ b_in, size_t b_stride, float* __restrict__ beta,
                                   float q_scale, float unit_eps) {
   const int t = blockIdx.x;
   const int lane = threadIdx.x & (RB_WAVE - 1);
   const int wave = threadIdx.x / RB_WAVE, n_waves = blockDim.x / RB_WAVE;
   float* row = qk + (size_t)t * qk_stride;
-  for (int v = wave; v < 2 * n_kv; v += n_waves) {           // the q heads, then the k heads
-    float* p = row + (size_t)v * dim;
-    float ss = 0.f;
-    for (int i = lane; i < dim; i += RB_WAVE) ss = fmaf(p[i], p[i], ss);
-    ss = wave_sum(ss);
-    const float f = (v < n_kv ? q_scale : 1.0f) / sqrtf(ss + unit_eps);
-    for (int i = lane; i < dim; i += RB_WAVE) p[i] *= f;
+  if (unit) {
+    for (int v = wave; v < 2 * n_kv; v += n_waves) {           // the q heads, then the k heads
+      float* p = row + (size_t)v * dim;
+      float ss = 0.f;
+      for (int i = lane; i < dim; i += RB_WAVE) ss = fmaf(p[i], p[i], ss);
+      ss = wave_sum(ss);
+      const float f = (v < n_kv ? q_scale : 1.0f) / sqrtf(ss + unit_eps);
+      for (int i = lane; i < dim; i += RB_WAVE) p[i] *= f;
+    }
+  } else if (q_scale != 1.0f) {
+    for (int i = threadIdx.x; i < n_kv * dim; i += blockDim.x) row[i] *= q_scale;
   }
   float* ar = a + (size_t)t * a_stride;
-  for (int i = threadIdx.x; i < n_heads * dim; i += blockDim.x) {
-    const int h = i / dim;
-    ar[i] = expf(-expf(a_log[h]) * rb_softplus(ar[i] + dt_bias[i]));
+  const int per_head = a_cols / n_heads;
+  for (int i = threadIdx.x; i < a_cols; i += blockDim.x) {
+    const float z = ar[i] + (bias ? bias[i] : 0.f);
+    if (decay == 0)
+      ar[i] = expf(-expf(a_log[i / per_head]) * rb_softplus(z));
+    else
+      ar[i] = expf(-rb_softplus(-z) / tau);
   }
-  for (int h = threadIdx.x; h < n_heads; h += blockDim.x) beta[(size_t)t * n_heads + h] = rb_sigmoid(b_in[(size_t)t * b_stride + h]);
+  if (b_in)
+    for (int h = threadIdx.x; h < n_heads; h += blockDim.x) beta[(size_t)t * n_heads + h] = rb_sigmoid(b_in[(size_t)t * b_stride + h]);
 }
 
+extern "C" int rb_recurrence_prep(float* qk, long long qk_stride, int n_kv_heads, int dim, int unit, float q_scale, float unit_eps,
+                                  float* a, long long a_stride, int a_cols, int decay, const float* bias, const float* a_log,
+                                  float tau, int n_heads, const float* b_in, long long b_stride, float* beta, int n_tokens,
+                                  void* stream) {
+  RB_RECORDED(rb_recurrence_prep(qk, qk_stride, n_kv_heads, dim, unit, q_scale, unit_eps, a, a_stride, a_cols, decay, bias, a_log,
+                                 tau, n_heads, b_in, b_stride, beta, n_tokens, stream));
+  RB_REQUIRE(n_tokens >= 0 && n_kv_heads > 0 && n_heads > 0 && dim > 0, "rb_recurrence_prep: bad sizes");
+  RB_REQUIRE(a_cols == n_heads || a_cols == n_heads * dim, "rb_recurrence_prep: %d decays a token for %d heads of %d", a_cols,
+             n_heads, dim);
+  RB_REQUIRE(qk_stride >= 2LL * n_kv_heads * dim && a_stride >= a_cols && (b_in == nullptr || b_stride >= n_heads),
+             "rb_recurrence_prep: a row stride is too short");
+  RB_REQUIRE((decay == 0 && a_log != nullptr) || (decay == 1 && tau > 0.f), "rb_recurrence_prep: decay %d lacks its constants", decay);
+  RB_REQUIRE(b_in == nullptr || beta != nullptr, "rb_recurrence_prep: beta has nowhere to go");
+  if (n_tokens == 0) return 0;
+  // a step of few tokens has few workgroups, and a token's heads are a chain of trips to memory for each wave: more waves then
+  const int threads = n_tokens < 2 * rb_compute_units() ? 1024 : 256;
+  recurrence_prep_kernel<<<n_tokens, threads, 0, (hipStream_t)stream>>>(qk, (size_t)qk_stride, n_kv_heads, dim, unit, a, (size_t)a_stride,
+                                                                    a_cols, decay, bias, a_log, tau, n_heads, b_in, (size_t)b_stride,
+                                                                    beta, q_scale, unit_eps);
+  RB_LAUNCH_CHECK();
+  return 0;
+}
+
+// The gated delta rule with a decay per key channel: unit vectors, decay 0 on H * dim numbers, beta.
 extern "C" int rb_delta_prep(float* qk, long long qk_stride, int n_kv_heads, int dim, float* a, long long a_stride, const float* dt_bias,
                              const float* a_log, int n_heads, const float* b_in, long long b_stride, float* beta,
                              float q_scale, float unit_eps, int n_tokens, void* stream) {
   RB_RECORDED(rb_delta_prep(qk, qk_stride, n_kv_heads, dim, a, a_stride, dt_bias, a_log, n_heads, b_in, b_stride, beta, q_scale,
                             unit_eps, n_tokens, stream));
-  RB_REQUIRE(n_tokens >= 0 && n_kv_heads > 0 && n_heads > 0 && dim > 0, "rb_delta_prep: bad sizes");
-  RB_REQUIRE(qk_stride >= 2LL * n_kv_heads * dim && b_stride >= n_heads && a_stride >= (long long)n_heads * dim,
-             "rb_delta_prep: a row stride is too short");
-  if (n_tokens == 0) return 0;
-  // a step of few tokens has few workgroups, and a token's heads are a chain of trips to memory for each wave: more waves then
-  const int threads = n_tokens < 2 * rb_compute_units() ? 1024 : 256;
-  delta_prep_kernel<<<n_tokens, threads, 0, (hipStream_t)stream>>>(qk, (size_t)qk_stride, n_kv_heads, dim, a, (size_t)a_stride, dt_bias, a_log,
-                                                               n_heads, b_in, (size_t)b_stride, beta, q_scale, unit_eps);
-  RB_LAUNCH_CHECK();
-  return 0;
+  return rb_recurrence_prep(qk, qk_stride, n_kv_heads, dim, 1, q_scale, unit_eps, a, a_stride, n_heads * dim, 0, dt_bias, a_log, 1.0f,
+                            n_heads, b_in, b_stride, beta, n_tokens, stream);
 }
 
 // ---------------------------------------------------------------- gated delta rule: the recurrence
@@ -201,7 +231,7 @@ __global__ __launch_bounds__(RB_WAVE) void delta_rule_kernel(
     const float* __restrict__ q, const float* __restrict__ k, size_t qk_stride, const float* __restrict__ v,
     size_t v_stride, const float* __restrict__ g, size_t g_stride, const float* __restrict__ beta, float* __restrict__ state,
     const int32_t* __restrict__ cu_seqlens, const int32_t* __restrict__ slots, float* __restrict__ out, int n_heads,
-    int n_kv, int dim, int vdim) {
+    int n_kv, int dim, int vdim, int g_per_head) {
   constexpr int COLS = RB_WAVE / RG;
   constexpr int DK = DKL * RG;               // rows held, >= dim; rows beyond dim stay zero
   constexpr int NQ = DK * CH / RB_WAVE;      // q (or k, or g) values of a chunk per lane
@@ -247,14 +277,14 @@ __global__ __launch_bounds__(RB_WAVE) void delta_rule_kernel(
       const size_t t = (size_t)(row0 + t0 + tt);
       rq[j] = in ? q[t * qk_stride + (size_t)kvh * dim + i] : 0.f;
       rk[j] = in ? k[t * qk_stride + (size_t)kvh * dim + i] : 0.f;
-      rgt[j] = in ? g[t * g_stride + (size_t)h * dim + i] : 0.f;
+      rgt[j] = in ? (g_per_head ? g[t * g_stride + h] : g[t * g_stride + (size_t)h * dim + i]) : 0.f;
     }
 #pragma unroll
     for (int j = 0; j < NV; ++j) {
       const int e = lane + RB_WAVE * j, tt = e / COLS, c = e - tt * COLS;
       rv[j] = (tt < nt && col0 + c < vdim) ? v[(size_t)(row0 + t0 + tt) * v_stride + (size_t)h * vdim + col0 + c] : 0.f;
     }
-    rb = lane < nt ? beta[(size_t)(row0 + t0 + lane) * n_heads + h] : 0.f;
+    rb = (beta && lane < nt) ? beta[(size_t)(row0 + t0 + lane) * n_heads + h] : 0.f;
   };
   if (n > 0) fetch(0);
   for (int t0 = 0; t0 < n; t0 += CH) {
@@ -299,7 +329,7 @@ __global__ __launch_bounds__(RB_WAVE) void delta_rule_kernel(
       const float kv = lanes_sum<RG>(kv0 + kv1);
       const float dq = lanes_sum<RG>(dq0 + dq1);
       const float kq = lanes_sum<RG>(kq0 + kq1);
-      const float u = bt * (vv - kv);
+      const float u = beta ? bt * (vv - kv) : vv;       // without beta: the plain rule, S <- diag(g) S + k v^T
 #pragma unroll
       for (int i = 0; i < DKL; ++i) s[i] = fmaf(sk[tt][rg * DKL + i], u, s[i]);
       if (rg == 0) so[tt][lane / RG] = fmaf(u, kq, dq);
@@ -336,12 +366,12 @@ template <int DKL, int RG, int CH>
 static void launch_delta_rule(const float* q, const float* k, size_t qk_stride, const float* v, size_t v_stride,
                               const float* g, size_t g_stride, const float* beta, float* state, const int32_t* cu_seqlens,
                               const int32_t* slots, float* out, int n_seqs, int n_heads, int n_kv, int dim, int vdim,
-                              hipStream_t s) {
+                              int g_per_head, hipStream_t s) {
   constexpr int COLS = RB_WAVE / RG;
   static_assert((DKL * RG * CH) % RB_WAVE == 0 && CH <= RB_WAVE && DKL % 4 == 0, "a chunk's values are dealt evenly to the lanes");
   dim3 grid(n_seqs, n_heads, (vdim + COLS - 1) / COLS);
   delta_rule_kernel<DKL, RG, CH><<<grid, RB_WAVE, 0, s>>>(q, k, qk_stride, v, v_stride, g, g_stride, beta, state, cu_seqlens,
-                                                          slots, out, n_heads, n_kv, dim, vdim);
+                                                          slots, out, n_heads, n_kv, dim, vdim, g_per_head);
 }
 
 extern "C" int rb_delta_rule(const float* q, const float* k, long long qk_stride, const float* v, long long v_stride,
@@ -350,11 +380,22 @@ extern "C" int rb_delta_rule(const float* q, const float* k, long long qk_stride
                              int vdim, void* stream) {
   RB_RECORDED(rb_delta_rule(q, k, qk_stride, v, v_stride, g, g_stride, beta, state, cu_seqlens, slots, out, n_seqs, n_tokens,
                             n_heads, n_kv_heads, dim, vdim, stream));
+  RB_REQUIRE(beta != nullptr, "rb_delta_rule: the delta rule needs beta");
+  return rb_linear_recurrence(q, k, qk_stride, v, v_stride, g, g_stride, 0, beta, state, cu_seqlens, slots, out, n_seqs, n_tokens,
+                              n_heads, n_kv_heads, dim, vdim, stream);
+}
+
+extern "C" int rb_linear_recurrence(const float* q, const float* k, long long qk_stride, const float* v, long long v_stride,
+                                    const float* g, long long g_stride, int g_per_head, const float* beta, float* state,
+                                    const int32_t* cu_seqlens, const int32_t* slots, float* out, int n_seqs, int n_tokens,
+                                    int n_heads, int n_kv_heads, int dim, int vdim, void* stream) {
+  RB_RECORDED(rb_linear_recurrence(q, k, qk_stride, v, v_stride, g, g_stride, g_per_head, beta, state, cu_seqlens, slots, out, n_seqs,
+                                   n_tokens, n_heads, n_kv_heads, dim, vdim, stream));
   RB_REQUIRE(n_seqs >= 0 && n_heads > 0 && n_kv_heads > 0 && n_heads % n_kv_heads == 0 && dim > 0 && vdim > 0,
-             "rb_delta_rule: bad sizes H=%d Hk=%d dim=%d vdim=%d", n_heads, n_kv_heads, dim, vdim);
-  RB_REQUIRE(g_stride >= (long long)n_heads * dim, "rb_delta_rule: the decays' row stride is too short");
-  RB_REQUIRE(dim <= 512, "rb_delta_rule: key size %d not supported (at most 512)", dim);
-  RB_REQUIRE(n_heads <= 65535 && vdim <= 65535 * 4, "rb_delta_rule: too many heads or value channels");
+             "rb_linear_recurrence: bad sizes H=%d Hk=%d dim=%d vdim=%d", n_heads, n_kv_heads, dim, vdim);
+  RB_REQUIRE(g_stride >= (long long)n_heads * (g_per_head ? 1 : dim), "rb_linear_recurrence: the decays' row stride is too short");
+  RB_REQUIRE(dim <= 512, "rb_linear_recurrence: key size %d not supported (at most 512)", dim);
+  RB_REQUIRE(n_heads <= 65535 && vdim <= 65535 * 4, "rb_linear_recurrence: too many heads or value channels");
   if (n_seqs == 0) return 0;
   hipStream_t s = (hipStream_t)stream;
   const size_t qs = (size_t)qk_stride, vs = (size_t)v_stride;
@@ -366,10 +407,10 @@ extern "C" int rb_delta_rule(const float* q, const float* k, long long qk_stride
     constexpr int CH1 = (DKL * RG >= RB_WAVE) ? 1 : RB_WAVE / (DKL * RG);                                                   \
     if (single)                                                                                                             \
       launch_delta_rule<DKL, RG, CH1>(q, k, qs, v, vs, g, (size_t)g_stride, beta, state, cu_seqlens, slots, out, n_seqs,   \
-                                      n_heads, n_kv_heads, dim, vdim, s);                                                   \
+                                      n_heads, n_kv_heads, dim, vdim, g_per_head, s);                                       \
     else                                                                                                                    \
       launch_delta_rule<DKL, RG, CH>(q, k, qs, v, vs, g, (size_t)g_stride, beta, state, cu_seqlens, slots, out, n_seqs,    \
-                                     n_heads, n_kv_heads, dim, vdim, s);                                                    \
+                                     n_heads, n_kv_heads, dim, vdim, g_per_head, s);                                        \
   } while (0)
   // Rows of a column over RG lanes, chunks as long as the registers that hold the next one allow.  A token's time is
   // its lane's share of the column, so while the waves do not fill the GPU's SIMDs a column goes to more lanes
@@ -401,7 +442,7 @@ extern "C" int rb_delta_rule(const float* q, const float* k, long long qk_stride
 template <typename TO>
 __global__ void gated_rmsnorm_kernel(const float* __restrict__ o, const float* __restrict__ weight,
                                      const float* __restrict__ gate, size_t gate_stride, float eps, TO* __restrict__ out,
-                                     int n_heads, int vdim, long long n_pairs) {
+                                     int n_heads, int vdim, long long n_pairs, int act) {
   const long long pair = (long long)blockIdx.x * (blockDim.x / RB_WAVE) + threadIdx.x / RB_WAVE;
   if (pair >= n_pairs) return;
   const int lane = threadIdx.x & (RB_WAVE - 1);
@@ -414,22 +455,29 @@ __global__ void gated_rmsnorm_kernel(const float* __restrict__ o, const float* _
   ss = wave_sum(ss);
   const float f = 1.0f / sqrtf(ss / (float)vdim + eps);
   for (int i = lane; i < vdim; i += RB_WAVE)
-    Num<TO>::store(out + (size_t)pair * vdim + i, p[i] * f * weight[i] * rb_sigmoid(gp[i]));
+    Num<TO>::store(out + (size_t)pair * vdim + i, p[i] * f * weight[i] * (act == 1 ? gp[i] * rb_sigmoid(gp[i]) : rb_sigmoid(gp[i])));
 }
 
 extern "C" int rb_gated_rmsnorm(const float* o, const float* weight, const float* gate, long long gate_stride, float eps,
                                 void* out, int out_dtype, int n_tokens, int n_heads, int vdim, void* stream) {
   RB_RECORDED(rb_gated_rmsnorm(o, weight, gate, gate_stride, eps, out, out_dtype, n_tokens, n_heads, vdim, stream));
-  RB_REQUIRE(n_tokens >= 0 && n_heads > 0 && vdim > 0, "rb_gated_rmsnorm: bad sizes");
+  return rb_gated_rmsnorm_act(o, weight, gate, gate_stride, 0, eps, out, out_dtype, n_tokens, n_heads, vdim, stream);
+}
+
+// act 0: the gate is sigmoid(gate); 1: silu(gate) = gate * sigmoid(gate)
+extern "C" int rb_gated_rmsnorm_act(const float* o, const float* weight, const float* gate, long long gate_stride, int act, float eps,
+                                    void* out, int out_dtype, int n_tokens, int n_heads, int vdim, void* stream) {
+  RB_RECORDED(rb_gated_rmsnorm_act(o, weight, gate, gate_stride, act, eps, out, out_dtype, n_tokens, n_heads, vdim, stream));
+  RB_REQUIRE(n_tokens >= 0 && n_heads > 0 && vdim > 0 && (act == 0 || act == 1), "rb_gated_rmsnorm: bad sizes");
   RB_REQUIRE(gate_stride >= (long long)n_heads * vdim, "rb_gated_rmsnorm: the gate's row stride is too short");
   if (n_tokens == 0) return 0;
   const long long n_pairs = (long long)n_tokens * n_heads;
   const int grid = (int)((n_pairs + 3) / 4);
   hipStream_t s = (hipStream_t)stream;
   if (out_dtype == RB_F32)
-    gated_rmsnorm_kernel<float><<<grid, 256, 0, s>>>(o, weight, gate, (size_t)gate_stride, eps, (float*)out, n_heads, vdim, n_pairs);
+    gated_rmsnorm_kernel<float><<<grid, 256, 0, s>>>(o, weight, gate, (size_t)gate_stride, eps, (float*)out, n_heads, vdim, n_pairs, act);
   else if (out_dtype == RB_BF16)
-    gated_rmsnorm_kernel<bf16_t><<<grid, 256, 0, s>>>(o, weight, gate, (size_t)gate_stride, eps, (bf16_t*)out, n_heads, vdim, n_pairs);
+    gated_rmsnorm_kernel<bf16_t><<<grid, 256, 0, s>>>(o, weight, gate, (size_t)gate_stride, eps, (bf16_t*)out, n_heads, vdim, n_pairs, act);
   else
     RB_REQUIRE(false, "rb_gated_rmsnorm: unknown dtype %d", out_dtype);
   RB_LAUNCH_CHECK();

@@ -22,7 +22,8 @@ __global__ void streams_layernorm_kernel(float* __restrict__ x, int n_streams, s
                                          const float* __restrict__ weight, const float* __restrict__ bias, float eps,
                                          const int32_t* __restrict__ rows, int width, TO* __restrict__ out,
                                          const float* __restrict__ mix, const float* __restrict__ out_coef,
-                                         const float* __restrict__ y, const float* __restrict__ scale) {
+                                         const float* __restrict__ y, const float* __restrict__ scale,
+                                         const float* __restrict__ delta2, float dscale) {
   extern __shared__ float u[];
   __shared__ float scratch[16];
   const int r = blockIdx.x;
@@ -56,7 +57,7 @@ __global__ void streams_layernorm_kernel(float* __restrict__ x, int n_streams, s
         v = coef ? fmaf(coef[s], xv, v) : v + xv;
       }
     }
-    if (delta) v += delta[src * width + j];
+    if (delta) v = fmaf(dscale, delta2 ? delta[src * width + j] + delta2[src * width + j] : delta[src * width + j], v);
     if (write_back) x[src * width + j] = v;
     u[j] = v;
     sum += v;
@@ -92,7 +93,7 @@ __global__ __launch_bounds__(1024) void streams_layernorm_vec_kernel(
     float* __restrict__ x, int n_streams, size_t stream_stride, const float* __restrict__ coef, const float* __restrict__ delta,
     const float* __restrict__ weight, const float* __restrict__ bias, float eps, const int32_t* __restrict__ rows, int width,
     TO* __restrict__ out, const float* __restrict__ mix, const float* __restrict__ out_coef, const float* __restrict__ y,
-    const float* __restrict__ scale) {
+    const float* __restrict__ scale, const float* __restrict__ delta2, float dscale) {
   extern __shared__ float u[];
   __shared__ float scratch[16];
   __shared__ float c_mix[ST_MAX_STREAMS * ST_MAX_STREAMS], c_out[ST_MAX_STREAMS], c_in[ST_MAX_STREAMS];
@@ -136,8 +137,12 @@ __global__ __launch_bounds__(1024) void streams_layernorm_vec_kernel(
         if (s < n_streams) v = fma4(c_in[s], ld4(x + (size_t)s * stream_stride + src * width + j), v);
     }
     if (delta) {
-      const float4 d = ld4(delta + src * width + j);
-      v = make_float4(v.x + d.x, v.y + d.y, v.z + d.z, v.w + d.w);
+      float4 d = ld4(delta + src * width + j);
+      if (delta2) {
+        const float4 e = ld4(delta2 + src * width + j);
+        d = make_float4(d.x + e.x, d.y + e.y, d.z + e.z, d.w + e.w);
+      }
+      v = fma4(dscale, d, v);
     }
     if (write_back) *reinterpret_cast<float4*>(x + src * width + j) = v;
     *reinterpret_cast<float4*>(u + j) = v;
@@ -182,6 +187,11 @@ extern "C" int rb_streams_layernorm(float* x, int n_streams, long long stream_st
 // The same after an update of the copies that was still to be done (rb_streams_update's mix, out_coef, y, scale; mix
 // null: none), in one pass over the rows: the copies are rewritten and the norm reads the new ones.  With an update
 // every row is taken (rows must be null).
+static int layernorm_launch(float* x, int n_streams, long long stream_stride, const float* mix, const float* out_coef, const float* y,
+                            const float* scale, const float* coef, const float* delta, const float* delta2, float dscale,
+                            const float* weight, const float* bias, float eps, const int32_t* rows, int n_rows, int width, void* out,
+                            int out_dtype, void* stream);
+
 extern "C" int rb_streams_update_layernorm(float* x, int n_streams, long long stream_stride, const float* mix,
                                            const float* out_coef, const float* y, const float* scale, const float* coef,
                                            const float* delta, const float* weight, const float* bias, float eps,
@@ -189,6 +199,26 @@ extern "C" int rb_streams_update_layernorm(float* x, int n_streams, long long st
                                            void* stream) {
   RB_RECORDED(rb_streams_update_layernorm(x, n_streams, stream_stride, mix, out_coef, y, scale, coef, delta, weight, bias, eps,
                                           rows, n_rows, width, out, out_dtype, stream));
+  return layernorm_launch(x, n_streams, stream_stride, mix, out_coef, y, scale, coef, delta, nullptr, 1.0f, weight, bias, eps, rows,
+                          n_rows, width, out, out_dtype, stream);
+}
+
+// Layer norm of a plain stream x [T, E] with the residual sum that was still to be done, in one pass:
+//   v = x[src] + dscale * (delta[src] + (delta2 ? delta2[src] : 0)),  src = rows ? rows[r] : r;  without rows x[src] = v as well;
+//   out[r] = (v - mean) / sqrt(var + eps) * weight + bias.   delta null: the norm alone.
+extern "C" int rb_layernorm_residual(float* x, const float* delta, const float* delta2, float dscale, const float* weight,
+                                     const float* bias, float eps, const int32_t* rows, int n_rows, int width, void* out,
+                                     int out_dtype, void* stream) {
+  RB_RECORDED(rb_layernorm_residual(x, delta, delta2, dscale, weight, bias, eps, rows, n_rows, width, out, out_dtype, stream));
+  RB_REQUIRE(delta != nullptr || delta2 == nullptr, "rb_layernorm_residual: a second term without a first");
+  return layernorm_launch(x, 1, 0, nullptr, nullptr, nullptr, nullptr, nullptr, delta, delta2, dscale, weight, bias, eps, rows, n_rows,
+                          width, out, out_dtype, stream);
+}
+
+static int layernorm_launch(float* x, int n_streams, long long stream_stride, const float* mix, const float* out_coef, const float* y,
+                            const float* scale, const float* coef, const float* delta, const float* delta2, float dscale,
+                            const float* weight, const float* bias, float eps, const int32_t* rows, int n_rows, int width, void* out,
+                            int out_dtype, void* stream) {
   RB_REQUIRE(mix == nullptr || (rows == nullptr && out_coef != nullptr && y != nullptr),
              "rb_streams_update_layernorm: an update takes every row and needs out_coef and y");
   RB_REQUIRE(n_rows >= 0 && width > 0 && width <= 16384, "rb_streams_layernorm: bad sizes %d x %d (width at most 16384)", n_rows, width);
@@ -198,25 +228,25 @@ extern "C" int rb_streams_update_layernorm(float* x, int n_streams, long long st
   hipStream_t s = (hipStream_t)stream;
   const size_t lds = (size_t)width * sizeof(float);
   auto aligned = [](const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; };
-  if (width % 4 == 0 && stream_stride % 4 == 0 && aligned(x) && aligned(delta) && aligned(weight) && aligned(bias) && aligned(out) &&
+  if (width % 4 == 0 && stream_stride % 4 == 0 && aligned(x) && aligned(delta) && aligned(delta2) && aligned(weight) && aligned(bias) && aligned(out) &&
       aligned(y) && aligned(scale) && (out_dtype == RB_F32 || out_dtype == RB_BF16)) {
     int threads = ((width / 4 + RB_WAVE - 1) / RB_WAVE) * RB_WAVE;
     if (threads > 1024) threads = 1024;
     if (out_dtype == RB_F32)
       streams_layernorm_vec_kernel<float><<<n_rows, threads, lds, s>>>(x, n_streams, (size_t)stream_stride, coef, delta, weight, bias,
-                                                                       eps, rows, width, (float*)out, mix, out_coef, y, scale);
+                                                                       eps, rows, width, (float*)out, mix, out_coef, y, scale, delta2, dscale);
     else
       streams_layernorm_vec_kernel<bf16_t><<<n_rows, threads, lds, s>>>(x, n_streams, (size_t)stream_stride, coef, delta, weight,
-                                                                        bias, eps, rows, width, (bf16_t*)out, mix, out_coef, y, scale);
+                                                                        bias, eps, rows, width, (bf16_t*)out, mix, out_coef, y, scale, delta2, dscale);
     RB_LAUNCH_CHECK();
     return 0;
   }
   if (out_dtype == RB_F32)
     streams_layernorm_kernel<float><<<n_rows, 256, lds, s>>>(x, n_streams, (size_t)stream_stride, coef, delta, weight, bias, eps,
-                                                             rows, width, (float*)out, mix, out_coef, y, scale);
+                                                             rows, width, (float*)out, mix, out_coef, y, scale, delta2, dscale);
   else if (out_dtype == RB_BF16)
     streams_layernorm_kernel<bf16_t><<<n_rows, 256, lds, s>>>(x, n_streams, (size_t)stream_stride, coef, delta, weight, bias, eps,
-                                                              rows, width, (bf16_t*)out, mix, out_coef, y, scale);
+                                                              rows, width, (bf16_t*)out, mix, out_coef, y, scale, delta2, dscale);
   else
     RB_REQUIRE(false, "rb_streams_layernorm: unknown dtype %d", out_dtype);
   RB_LAUNCH_CHECK();

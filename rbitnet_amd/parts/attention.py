@@ -12,7 +12,18 @@ on top of any past.
 Parameters: num_heads, num_kv_heads, head_dim, scale, window (None: all keys; n: the
 last n keys including the token's own), position (a PartSpec), cache_from (None, or the
 index of the layer whose cache this layer reads instead of keeping one), names (tensor
-names of the four matrices relative to the layer's prefix).
+names of the matrices relative to the layer's prefix), and three that a plain decoder leaves out:
+  value_dim   size of a value head where it is not head_dim;
+  sink        True: a learned number per query head (tensor "sink") stands in the softmax's
+              denominator as exp(sink): no key, no value, not scaled;
+  head_gate   True: head h's output is multiplied by sigmoid(Wg h)_h (tensor "gate" [heads, E])
+              before the output matrix.
+A position part that rotates only the first numbers of a head says so with its own head_dim
+(the table's width).  Where keys and values differ in size, or only a part of a head is
+rotated, queries, keys and values are laid out with one head size, the larger of the two,
+the rest being zeros: the scores and the sums stay what they are and every attention kernel
+made for one head size serves (keys of 64 beside values of 128 cost a third more cache
+traffic than their own sizes would).
 
 Interface of a mixer:
   tensor_specs() / load(tensors)
@@ -34,7 +45,8 @@ from ..errors import ConfigError
 from .base import BuildEnv, CacheRequest, Part, TensorSpec, build_part, register_mixer
 from .linear import linear, linear_or_terms, linear_to_stream, pack_rows
 
-DEFAULT_NAMES = {"q": "q_proj.weight", "k": "k_proj.weight", "v": "v_proj.weight", "o": "o_proj.weight"}
+DEFAULT_NAMES = {"q": "q_proj.weight", "k": "k_proj.weight", "v": "v_proj.weight", "o": "o_proj.weight", "sink": "sink",
+                 "gate": "gate"}
 _MATRIX_CORE_HEAD_DIMS = (64, 128)
 _DECODE_GROUPS = tuple(range(1, 17))    # query heads per kv head the decode kernels take
 
@@ -54,6 +66,10 @@ class Attention(Part):
             raise ConfigError(f"attention: {self.n_heads} heads cannot share {self.n_kv} kv heads")
         if self.head_dim <= 0 or self.head_dim % 2 != 0 or self.head_dim > 256:
             raise ConfigError(f"attention: head_dim {self.head_dim} not supported (even, at most 256)")
+        self.value_dim = int(params.get("value_dim") or self.head_dim)
+        if not 0 < self.value_dim <= 512:
+            raise ConfigError(f"attention: value_dim {self.value_dim} not supported (1 to 512)")
+        self.has_sink, self.has_gate = bool(params.get("sink")), bool(params.get("head_gate"))
         self.scale = float(params.get("scale") or self.head_dim ** -0.5)
         self.window = params.get("window")
         if self.window is not None and int(self.window) <= 0:
@@ -63,6 +79,15 @@ class Attention(Part):
         self.position = build_part("position", params["position"], env)
         self.plan_safe = bool(getattr(self.position, "plan_safe", False))
         self.hidden = env.hidden_size
+        # how many numbers of a head the position part rotates (its table's width; none: 0), and the one head size
+        # that queries, keys and values are laid out with
+        self.rot = int(getattr(self.position, "head_dim", 0)) if getattr(self.position, "rotation_tables", None) else 0
+        if self.rot > self.head_dim:
+            raise ConfigError(f"attention: {self.rot} rotated numbers in a head of {self.head_dim}")
+        self.pad = max(self.head_dim, self.value_dim)
+        self.same_sizes = self.value_dim == self.head_dim and self.rot in (0, self.head_dim)
+        self.w_gate = None
+        self.sink: Optional[torch.Tensor] = None
         self.w_qkv: Optional[torch.Tensor] = None
         self.w_q: Optional[torch.Tensor] = None
         self.w_o: Optional[torch.Tensor] = None
@@ -70,10 +95,15 @@ class Attention(Part):
     # ------------------------------------------------------------------ tensors
     def tensor_specs(self) -> Dict[str, TensorSpec]:
         qd, kd = self.n_heads * self.head_dim, self.n_kv * self.head_dim
-        specs = {self.names["q"]: TensorSpec((qd, self.hidden)), self.names["o"]: TensorSpec((self.hidden, qd))}
+        specs = {self.names["q"]: TensorSpec((qd, self.hidden)),
+                 self.names["o"]: TensorSpec((self.hidden, self.n_heads * self.value_dim))}
         if self.cache_from is None:
             specs[self.names["k"]] = TensorSpec((kd, self.hidden))
-            specs[self.names["v"]] = TensorSpec((kd, self.hidden))
+            specs[self.names["v"]] = TensorSpec((self.n_kv * self.value_dim, self.hidden))
+        if self.has_sink:
+            specs[self.names["sink"]] = TensorSpec((self.n_heads,), role="gain", init="normal")
+        if self.has_gate:
+            specs[self.names["gate"]] = TensorSpec((self.n_heads, self.hidden))
         return specs
 
     def load(self, tensors: Dict[str, torch.Tensor]) -> None:
@@ -88,22 +118,43 @@ class Attention(Part):
         first = pieces[0][0]
         self.w_qkv = pack_rows(lib, pieces, row, self.hidden, first.dtype, first.device, allowed)
         o = tensors[self.names["o"]]
+        if self.value_dim < self.pad:
+            # attention's output comes in heads of `pad` numbers whose last ones are zero: columns of zeros for them
+            wide = torch.zeros((o.shape[0], self.n_heads, self.pad), dtype=o.dtype, device=o.device)
+            wide[:, :, :self.value_dim] = o.view(o.shape[0], self.n_heads, self.value_dim)
+            o = wide.view(o.shape[0], self.n_heads * self.pad)
         self.w_o = pack_rows(lib, [(o, 0, None, None)], o.shape[0], o.shape[1], o.dtype, o.device, allowed)
+        if self.has_sink:
+            self.sink = tensors[self.names["sink"]]
+        if self.has_gate:
+            # rows up to a multiple of 16 (zeros), so that the product's kernels find whole tiles
+            g = tensors[self.names["gate"]]
+            rows = (self.n_heads + 15) // 16 * 16
+            full = torch.zeros((rows, self.hidden), dtype=g.dtype, device=g.device)
+            full[:self.n_heads] = g
+            self.w_gate = pack_rows(lib, [(full, 0, None, None)], rows, self.hidden, g.dtype, g.device, allowed)
 
     def cache_request(self) -> Optional[CacheRequest]:
         if self.cache_from is not None:
             return None
-        return CacheRequest("kv", heads=self.n_kv, head_dim=self.head_dim,
+        return CacheRequest("kv", heads=self.n_kv, head_dim=self.pad,
                             window=None if self.window is None else int(self.window))
 
     # ------------------------------------------------------------------ forward
+    def _gate_and_project(self, attn, h, stream, next_norm):
+        lib = self.env.lib
+        if self.has_gate:
+            logits = linear(lib, h, self.w_gate, torch.float32)
+            lib.head_gate(attn, logits, 0, self.n_heads, self.pad)
+        return linear_to_stream(lib, attn, self.w_o, stream, next_norm)
+
     def forward(self, h, ctx, view, stream: Optional[torch.Tensor] = None, next_norm=None):
         lib = self.env.lib
         t = h.shape[0]
-        hq, hk, d = self.n_heads, self.n_kv, self.head_dim
+        hq, hk, d = self.n_heads, self.n_kv, self.pad
         owns = self.cache_from is None
         # q, k and v of the step; as the terms of the product where the position part reads such
-        if getattr(self.position, "takes_terms", False):
+        if self.same_sizes and getattr(self.position, "takes_terms", False):
             qkv = linear_or_terms(lib, h, self.w_qkv)
         else:
             qkv = linear(lib, h, self.w_qkv, torch.float32)
@@ -114,29 +165,36 @@ class Attention(Part):
                 and not getattr(self.env, "generic_only", False))
         decode = fast and ctx.max_q_len == 1 and (hq // hk) in _DECODE_GROUPS
         tables = getattr(self.position, "rotation_tables", None)
-        if decode and owns and tables is not None:
+        if decode and owns and tables is not None and self.same_sizes and not self.has_sink:
             # one kernel: rotation, cache write, attention over the pages
             cos, sin, style = tables()
             n_splits, workspace = ctx.decode_workspace(hq, d, hk)
             lib.attention_decode_fused_bf16(qkv, cos, sin, style, view.k_pages, view.v_pages, attn, ctx.tok_pos, bt,
                                             hq, hk, d, self.scale, window, n_splits, workspace)
-            return linear_to_stream(lib, attn, self.w_o, stream, next_norm)
+            return self._gate_and_project(attn, h, stream, next_norm)
         q = torch.empty((t, hq, d), dtype=self.env.dtype, device=h.device)
-        if owns:
-            self.position.encode_and_store(qkv, q, view.k_pages, view.v_pages, ctx, bt, hq, hk, d)
+        if self.same_sizes:
+            if owns:
+                self.position.encode_and_store(qkv, q, view.k_pages, view.v_pages, ctx, bt, hq, hk, d)
+            else:
+                self.position.encode_and_store(qkv, q, None, None, ctx, bt, hq, 0, d)
         else:
-            self.position.encode_and_store(qkv, q, None, None, ctx, bt, hq, 0, d)
+            cos, sin, style = tables() if self.rot else (None, None, 1)
+            if self.rot and style != 1:
+                raise ConfigError("attention: a head rotated in part pairs i with i + rot / 2 (style 'half')")
+            lib.rope_store(qkv, cos, sin, self.rot, q, view.k_pages if owns else None, view.v_pages if owns else None,
+                           ctx.tok_pos, ctx.tok_seq, bt, hq, hk, self.head_dim, self.value_dim, d)
         if decode:
             n_splits, workspace = ctx.decode_workspace(hq, d, hk)
             lib.attention_decode_bf16(q, view.k_pages, view.v_pages, attn, ctx.tok_pos, bt, hq, hk, d,
-                                      self.scale, window, n_splits, workspace)
+                                      self.scale, window, n_splits, workspace, sinks=self.sink)
         elif fast:
             lib.attention_prefill_bf16(q, view.k_pages, view.v_pages, attn, ctx.cu_seqlens, ctx.past_len, bt,
-                                       ctx.n_seqs, ctx.max_q_len, hq, hk, d, self.scale, window)
+                                       ctx.n_seqs, ctx.max_q_len, hq, hk, d, self.scale, window, sinks=self.sink)
         else:
-            lib.attention_generic(q, view.k_pages, view.v_pages, attn, ctx.tok_pos, ctx.tok_seq, bt, hq, hk, d,
-                                  self.scale, window)
-        return linear_to_stream(lib, attn, self.w_o, stream, next_norm)
+            lib.attention_sinks(q, view.k_pages, view.v_pages, attn, ctx.tok_pos, ctx.tok_seq, bt, hq, hk, d,
+                                self.scale, window, self.sink)
+        return self._gate_and_project(attn, h, stream, next_norm)
 
 
 register_mixer("attention", Attention)

@@ -23,7 +23,8 @@ from typing import Dict
 import torch
 
 from .base import BuildEnv, build_part, register_block
-from .stream import normed_for, sublayer  # noqa: F401  (normed_for: its old home)
+from ..errors import ConfigError
+from .stream import ScaledSum, normed_for, sublayer  # noqa: F401  (normed_for: its old home)
 
 DEFAULT_SEGMENTS = {"norm1": "input_layernorm", "mixer": "self_attn", "norm2": "post_attention_layernorm",
                     "feed_forward": "mlp"}
@@ -60,4 +61,58 @@ class PreNormBlock:
         return sublayer(self.feed_forward, self.norm2, x, a, next_norm, ctx)
 
 
+class ParallelBlock:
+    """"parallel": one norm that both sublayers read, and a factor m on their sum:
+        h = norm1(x);  x += m * (mixer(h) + feed_forward(h))
+    The feed-forward may be left out.  The sum is left to the norm that reads the stream next (`ScaledSum`), which adds
+    it in its own pass over the rows; that norm must say `adds_scaled_sum` (layer norm does).
+    Block parameters (`LayerSpec.params`): residual_scale (m, 1.0)."""
+    takes_next_norm = True
+
+    def __init__(self, layer_spec, env: BuildEnv):
+        params = dict(getattr(layer_spec, "params", None) or {})
+        self.scale = float(params.get("residual_scale", 1.0))
+        self.norm1 = build_part("norm", layer_spec.norm1, env)
+        self.mixer = build_part("mixer", layer_spec.mixer, env)
+        self.feed_forward = None if layer_spec.feed_forward is None else build_part("feed_forward", layer_spec.feed_forward, env)
+        self.segments = dict({"norm1": "norm1", "mixer": "mix", "feed_forward": "mlp"}, **(getattr(layer_spec, "segments", None) or {}))
+        if not getattr(self.norm1, "adds_scaled_sum", False):
+            raise ConfigError("a parallel layer needs a norm that adds a scaled sum in its own pass (layernorm)")
+
+    def _all(self):
+        return [p for p in (self.norm1, self.mixer, self.feed_forward) if p is not None]
+
+    @property
+    def graph_safe(self) -> bool:
+        return all(getattr(p, "graph_safe", False) for p in self._all())
+
+    @property
+    def plan_safe(self) -> bool:
+        return all(getattr(p, "plan_safe", False) for p in self._all())
+
+    def parts(self) -> Dict[str, object]:
+        out = {self.segments["norm1"]: self.norm1, self.segments["mixer"]: self.mixer}
+        if self.feed_forward is not None:
+            out[self.segments["feed_forward"]] = self.feed_forward
+        return out
+
+    def cache_requests(self):
+        many = getattr(self.mixer, "cache_requests", None)
+        one = getattr(self.mixer, "cache_request", None)
+        return list(many()) if many else ([one()] if one and one() is not None else [])
+
+    @property
+    def first_norm(self):
+        return self.norm1
+
+    def forward(self, x: torch.Tensor, pending, ctx, view, next_norm=None):
+        if next_norm is not None and not getattr(next_norm, "adds_scaled_sum", False):
+            raise ConfigError("what follows a parallel layer must begin with a norm that adds a scaled sum (layernorm)")
+        h = self.norm1.forward(x, pending, None)
+        a = self.mixer.forward(h, ctx, view)
+        b = self.feed_forward.forward(h, ctx) if self.feed_forward is not None else None
+        return ScaledSum(a, b, self.scale)
+
+
 register_block("prenorm", PreNormBlock)
+register_block("parallel", ParallelBlock)

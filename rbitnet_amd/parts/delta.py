@@ -123,4 +123,165 @@ class ChannelDelta(Part):
         return linear(lib, on, self.w_o, torch.float32)
 
 
+class HeadDelta(Part):
+    """The gated delta rule with ONE decay per head and a full gate on the read-out:
+        q, k, v as above (convolution, silu; q, k unit vectors, q times dim^(-1/2));  beta = sigmoid(Wb h)
+        g = exp(-exp(A_log[head]) * softplus(Wa h + dt_bias))                    one number per head
+        S <- g S;  u = beta (v - S^T k);  S <- S + k u^T;  o = S^T q
+        o <- o / sqrt(mean(o^2) + eps) * norm * silu(Wg h);   out = Wo o
+    All projections are one product; the recurrence is the same kernel with the decay read once per head.
+    Parameters: heads, kv_heads, dim, vdim, conv (taps), eps, unit_eps (1e-6), names."""
+    graph_safe = True
+    plan_safe = True
+
+    NAMES = {"q": "q", "k": "k", "v": "v", "q_conv": "q.conv", "k_conv": "k.conv", "v_conv": "v.conv", "b": "b", "a": "a",
+             "a_log": "A_log", "dt_bias": "dt_bias", "norm": "norm", "g": "g", "o": "o"}
+
+    def __init__(self, params: Dict, env: BuildEnv):
+        self.env = env
+        self.heads = int(params["heads"])
+        self.kv_heads = int(params.get("kv_heads") or self.heads)
+        self.dim, self.vdim = int(params["dim"]), int(params["vdim"])
+        self.taps = int(params["conv"])
+        self.eps = float(params["eps"])
+        self.unit_eps = float(params.get("unit_eps", 1e-6))
+        if self.heads <= 0 or self.kv_heads <= 0 or self.heads % self.kv_heads != 0:
+            raise ConfigError(f"delta rule: {self.heads} heads cannot share {self.kv_heads} q/k heads")
+        if not 0 < self.dim <= 512:
+            raise ConfigError(f"delta rule: key size {self.dim} not supported (1 to 512)")
+        self.names = dict(self.NAMES, **(params.get("names") or {}))
+        self.hidden = env.hidden_size
+        self.n_qk, self.n_v = self.kv_heads * self.dim, self.heads * self.vdim
+        self.n_conv = 2 * self.n_qk + self.n_v
+        self.conv = ShortConv(self.n_conv, self.taps, env, residual=False, act=ACT_SILU)
+        self.cache_from = None
+
+    def tensor_specs(self) -> Dict[str, TensorSpec]:
+        n, e = self.names, self.hidden
+        gain = lambda *shape: TensorSpec(tuple(shape), role="gain", init="normal")
+        return {
+            n["q"]: TensorSpec((self.n_qk, e)), n["k"]: TensorSpec((self.n_qk, e)), n["v"]: TensorSpec((self.n_v, e)),
+            n["q_conv"]: gain(self.n_qk, self.taps), n["k_conv"]: gain(self.n_qk, self.taps),
+            n["v_conv"]: gain(self.n_v, self.taps),
+            n["b"]: TensorSpec((self.heads, e)), n["a"]: TensorSpec((self.heads, e)),
+            n["a_log"]: gain(self.heads), n["dt_bias"]: gain(self.heads),
+            n["norm"]: TensorSpec((self.vdim,), role="gain", init="ones_normal"),
+            n["g"]: TensorSpec((self.n_v, e)), n["o"]: TensorSpec((e, self.n_v)),
+        }
+
+    def load(self, tensors: Dict[str, torch.Tensor]) -> None:
+        lib, allowed, n = self.env.lib, not getattr(self.env, "generic_only", False), self.names
+        first = tensors[n["q"]]
+        pieces, row = [], 0
+        self.cols = {}
+        for key in ("q", "k", "v", "b", "a", "g"):           # one product: [q | k | v | beta | decay | gate]
+            self.cols[key] = row
+            pieces.append((tensors[n[key]], row, None, None))
+            row += tensors[n[key]].shape[0]
+        self.w_in = pack_rows(lib, pieces, row, self.hidden, first.dtype, first.device, allowed)
+        self.conv.load(torch.cat([tensors[n["q_conv"]], tensors[n["k_conv"]], tensors[n["v_conv"]]]))
+        self.a_log, self.dt_bias, self.norm = tensors[n["a_log"]], tensors[n["dt_bias"]], tensors[n["norm"]]
+        o = tensors[n["o"]]
+        self.w_o = pack_rows(lib, [(o, 0, None, None)], o.shape[0], o.shape[1], o.dtype, o.device, allowed)
+
+    def cache_requests(self) -> List[CacheRequest]:
+        out = [CacheRequest("state", state_shape=(self.heads, self.vdim, self.dim), state_init=0.0, name="delta")]
+        conv = self.conv.cache_request("conv")
+        return out + ([conv] if conv else [])
+
+    def cache_request(self) -> Optional[CacheRequest]:
+        return self.cache_requests()[0]
+
+    def forward(self, h: torch.Tensor, ctx, view, stream: Optional[torch.Tensor] = None, next_norm=None) -> torch.Tensor:
+        lib, t, c = self.env.lib, h.shape[0], self.cols
+        proj = linear(lib, h, self.w_in, torch.float32)
+        qkv = self.conv.forward(proj, ctx, view.states.get("conv"), torch.float32)
+        beta = torch.empty((t, self.heads), dtype=torch.float32, device=h.device)
+        lib.recurrence_prep(qkv, self.kv_heads, self.dim, True, self.dim ** -0.5, self.unit_eps, proj, c["a"], self.heads, 0,
+                            self.dt_bias, self.a_log, 1.0, self.heads, b_in=proj, b_col=c["b"], beta=beta)
+        o = torch.empty((t, self.n_v), dtype=torch.float32, device=h.device)
+        lib.linear_recurrence(qkv, self.kv_heads, self.dim, self.heads, self.vdim, proj, c["a"], True, beta,
+                              view.states["delta"], ctx, o)
+        on = torch.empty((t, self.n_v), dtype=self.env.dtype, device=h.device)
+        lib.gated_rmsnorm_act(o, self.norm, proj, c["g"], 1, self.eps, self.heads, self.vdim, on)
+        return linear(lib, on, self.w_o, torch.float32)
+
+
+class DecayAttention(Part):
+    """Gated linear attention: a matrix state per head that decays per key channel and is read with the query.
+        q = Wq h * dim^(-1/2),  k = Wk h  (heads x dim);  v = Wv h  (heads x vdim)
+        alpha = sigmoid(Wa2 (Wa1 h) + bias) ^ (1 / tau)                          heads x dim, in float32
+        S <- diag(alpha) S + k v^T;  o = S^T q          (the plain rule: no correction towards the new value)
+        o <- o / sqrt(mean(o^2) + eps) * norm;  out = Wo (o * silu(Wg h))
+    The state lives in the cache's per-slot storage (`view.states["decay"]`, [slots, heads, vdim, dim] float32).
+    Parameters: heads, dim, vdim, tau, decay_rank (the inner size of the decay's two matrices), eps, names."""
+    graph_safe = True
+    plan_safe = True
+
+    NAMES = {"q": "q", "k": "k", "v": "v", "g": "g", "o": "o", "norm": "norm", "a1": "a1", "a2": "a2", "a_bias": "a2.b"}
+
+    def __init__(self, params: Dict, env: BuildEnv):
+        self.env = env
+        self.heads, self.dim, self.vdim = int(params["heads"]), int(params["dim"]), int(params["vdim"])
+        self.tau = float(params["tau"])
+        self.decay_rank = int(params["decay_rank"])
+        self.eps = float(params["eps"])
+        if min(self.heads, self.dim, self.vdim, self.decay_rank) <= 0 or self.dim > 512:
+            raise ConfigError("decay attention: sizes must be positive, the key size at most 512")
+        if not self.tau > 0:
+            raise ConfigError(f"decay attention: tau must be positive, found {self.tau}")
+        self.names = dict(self.NAMES, **(params.get("names") or {}))
+        self.hidden = env.hidden_size
+        self.n_qk, self.n_v = self.heads * self.dim, self.heads * self.vdim
+        self.cache_from = None
+
+    def tensor_specs(self) -> Dict[str, TensorSpec]:
+        n, e = self.names, self.hidden
+        return {
+            n["q"]: TensorSpec((self.n_qk, e)), n["k"]: TensorSpec((self.n_qk, e)), n["v"]: TensorSpec((self.n_v, e)),
+            n["g"]: TensorSpec((self.n_v, e)), n["o"]: TensorSpec((e, self.n_v)),
+            n["norm"]: TensorSpec((self.vdim,), role="gain", init="ones_normal"),
+            n["a1"]: TensorSpec((self.decay_rank, e)), n["a2"]: TensorSpec((self.n_qk, self.decay_rank)),
+            n["a_bias"]: TensorSpec((self.n_qk,), role="gain", init="normal"),
+        }
+
+    def load(self, tensors: Dict[str, torch.Tensor]) -> None:
+        lib, allowed, n = self.env.lib, not getattr(self.env, "generic_only", False), self.names
+        first = tensors[n["q"]]
+        pieces, row = [], 0
+        self.cols = {}
+        for key in ("q", "k", "v", "g"):                     # one product: [q | k | v | gate]
+            self.cols[key] = row
+            pieces.append((tensors[n[key]], row, None, None))
+            row += tensors[n[key]].shape[0]
+        self.w_in = pack_rows(lib, pieces, row, self.hidden, first.dtype, first.device, allowed)
+        a1, a2 = tensors[n["a1"]], tensors[n["a2"]]
+        self.w_a1 = pack_rows(lib, [(a1, 0, None, None)], a1.shape[0], a1.shape[1], a1.dtype, a1.device, allowed)
+        self.w_a2 = pack_rows(lib, [(a2, 0, None, None)], a2.shape[0], a2.shape[1], a2.dtype, a2.device, allowed)
+        self.a_bias, self.norm = tensors[n["a_bias"]], tensors[n["norm"]]
+        o = tensors[n["o"]]
+        self.w_o = pack_rows(lib, [(o, 0, None, None)], o.shape[0], o.shape[1], o.dtype, o.device, allowed)
+
+    def cache_requests(self) -> List[CacheRequest]:
+        return [CacheRequest("state", state_shape=(self.heads, self.vdim, self.dim), state_init=0.0, name="decay")]
+
+    def cache_request(self) -> Optional[CacheRequest]:
+        return self.cache_requests()[0]
+
+    def forward(self, h: torch.Tensor, ctx, view, stream: Optional[torch.Tensor] = None, next_norm=None) -> torch.Tensor:
+        lib, t, c, dt = self.env.lib, h.shape[0], self.cols, self.env.dtype
+        proj = linear(lib, h, self.w_in, torch.float32)                       # [T, q | k | v | gate]
+        low = linear(lib, h, self.w_a1, dt)
+        z = linear(lib, low, self.w_a2, torch.float32)                        # [T, heads * dim]
+        lib.recurrence_prep(proj, self.heads, self.dim, False, self.dim ** -0.5, 0.0, z, 0, self.n_qk, 1, self.a_bias, None,
+                            self.tau, self.heads)
+        o = torch.empty((t, self.n_v), dtype=torch.float32, device=h.device)
+        lib.linear_recurrence(proj, self.heads, self.dim, self.heads, self.vdim, z, 0, False, None, view.states["decay"], ctx, o)
+        on = torch.empty((t, self.n_v), dtype=dt, device=h.device)
+        lib.gated_rmsnorm_act(o, self.norm, proj, c["g"], 1, self.eps, self.heads, self.vdim, on)
+        return linear(lib, on, self.w_o, torch.float32)
+
+
 register_mixer("channel_delta", ChannelDelta)
+register_mixer("gated_delta", HeadDelta)
+register_mixer("decay_attention", DecayAttention)

@@ -24,7 +24,7 @@ from typing import Dict, Optional
 import torch
 
 from .base import BuildEnv, Part, TensorSpec, register_norm
-from .stream import GainedRows, StreamsUpdate  # noqa: F401  (GainedRows: its old home; importers find it here too)
+from .stream import GainedRows, ScaledSum, StreamsUpdate  # noqa: F401  (GainedRows: its old home; importers find it here too)
 
 
 class RMSNorm(Part):
@@ -60,6 +60,7 @@ class LayerNorm(Part):
     [S, T, E]: the norm then reads sum_s coef[s] x[s] (`coef` None: the plain sum)."""
     graph_safe = True
     plan_safe = True
+    adds_scaled_sum = True        # delta may be a ScaledSum: scale * (a + b), added in the norm's own pass
 
     def __init__(self, params: Dict, env: BuildEnv):
         self.size = int(params["size"])
@@ -89,6 +90,10 @@ class LayerNorm(Part):
         t = x.shape[-2]
         n = t if rows is None else rows.shape[0]
         out = torch.empty((n, self.size), dtype=out_dtype or self.env.dtype, device=x.device)
+        if isinstance(delta, ScaledSum):                  # a plain stream [T, E] and the residual sum that is still to be done
+            a, b, scale = delta.parts()
+            self.env.lib.layernorm_residual(x, a, b, scale, self.weight, self.bias, self.eps, rows, out)
+            return out
         update = None
         if isinstance(delta, StreamsUpdate):              # an update of the copies still to be done
             if rows is None:

@@ -1,0 +1,85 @@
+"""A feed-forward of many small experts of which every token uses a few.
+
+    z = W_router h (float32);  s = sigmoid(z);  the `top` experts with the largest s are chosen (lowest index among equals)
+    out = sum over the chosen e of expert_e(s_e * h): the score multiplies the expert's INPUT and is not renormalised
+    expert(x):  g = min(Wg x, limit),  u = clamp(Wu x, -limit, limit),  Wd (g * sigmoid(alpha * g) * (u + 1))
+
+Nothing of a step goes through the host: the router's product, one launch that chooses and sorts the (token, expert)
+pairs by expert in runs padded to tiles of 16 rows, one launch pair for all experts' products (on the matrix cores in
+bfloat16), and, with more than one expert a token, the sum of a token's pairs in a fixed order.  A token's result does
+not depend on what else the step holds.
+
+Experts' tensors are `e<i>.gate`, `e<i>.up` [ff, E] and `e<i>.down` [E, ff]; they are stacked at load time.
+Parameters: experts, top, intermediate_size, limit, alpha (1.702), names ({"router", "expert", "gate", "up", "down"}).
+"""
+from __future__ import annotations
+
+from typing import Dict, Optional
+
+import torch
+
+from ..errors import ConfigError
+from .base import BuildEnv, Part, TensorSpec, register_feed_forward
+from .linear import linear, pack_rows
+
+DEFAULT_NAMES = {"router": "router", "expert": "e{i}", "gate": "gate", "up": "up", "down": "down"}
+MAX_EXPERTS = 1024
+
+
+class RoutedExperts(Part):
+    graph_safe = True
+    plan_safe = True
+
+    def __init__(self, params: Dict, env: BuildEnv):
+        self.env = env
+        self.n_experts, self.top = int(params["experts"]), int(params["top"])
+        self.ff = int(params["intermediate_size"])
+        self.limit = float(params["limit"])
+        self.alpha = float(params.get("alpha", 1.702))
+        if not 0 < self.top <= self.n_experts <= MAX_EXPERTS:
+            raise ConfigError(f"routed experts: top {self.top} of {self.n_experts} experts not supported (at most {MAX_EXPERTS})")
+        if self.ff <= 0 or not self.limit > 0:
+            raise ConfigError("routed experts: sizes and the limit must be positive")
+        self.names = dict(DEFAULT_NAMES, **(params.get("names") or {}))
+        self.hidden = env.hidden_size
+
+    def _name(self, i: int, what: str) -> str:
+        return f"{self.names['expert'].format(i=i)}.{self.names[what]}"
+
+    def tensor_specs(self) -> Dict[str, TensorSpec]:
+        out = {self.names["router"]: TensorSpec((self.n_experts, self.hidden))}
+        for i in range(self.n_experts):
+            out[self._name(i, "gate")] = TensorSpec((self.ff, self.hidden))
+            out[self._name(i, "up")] = TensorSpec((self.ff, self.hidden))
+            out[self._name(i, "down")] = TensorSpec((self.hidden, self.ff))
+        return out
+
+    def load(self, tensors: Dict[str, torch.Tensor]) -> None:
+        lib, allowed = self.env.lib, not getattr(self.env, "generic_only", False)
+        r = tensors[self.names["router"]]
+        self.w_router = pack_rows(lib, [(r, 0, None, None)], r.shape[0], r.shape[1], r.dtype, r.device, allowed)
+        stack = lambda what: torch.stack([tensors[self._name(i, what)] for i in range(self.n_experts)]).contiguous()
+        self.w_gate, self.w_up, self.w_down = stack("gate"), stack("up"), stack("down")
+
+    def forward(self, h: torch.Tensor, ctx=None, stream: Optional[torch.Tensor] = None, next_norm=None) -> torch.Tensor:
+        lib, t, dev = self.env.lib, h.shape[0], h.device
+        z = linear(lib, h, self.w_router, torch.float32)
+        pairs = t * self.top
+        max_rows = lib.routed_rows(t, self.top, self.n_experts)
+        sel = torch.empty(pairs, dtype=torch.int32, device=dev)
+        weight = torch.empty(pairs, dtype=torch.float32, device=dev)
+        row_pair = torch.empty(max_rows, dtype=torch.int32, device=dev)
+        tile_expert = torch.empty(max_rows // 16, dtype=torch.int32, device=dev)
+        lib.route_top(z, self.n_experts, self.top, sel, weight, row_pair, tile_expert)
+        y = torch.empty((max_rows, self.ff), dtype=h.dtype, device=dev)
+        out = torch.empty((pairs, self.hidden), dtype=torch.float32, device=dev)
+        lib.routed_experts(h, weight, self.top, row_pair, tile_expert, self.w_gate, self.w_up, self.w_down, y, out,
+                           self.limit, self.alpha)
+        if self.top == 1:
+            return out
+        total = torch.empty((t, self.hidden), dtype=torch.float32, device=dev)
+        lib.pairs_sum(out, self.top, total)
+        return total
+
+
+register_feed_forward("routed_experts", RoutedExperts)

@@ -14,6 +14,8 @@ prepared for the norm that follows, `GainedRows`).  What a sublayer has not yet 
     GainedRows      nothing to add, and the rows as the next norm's kernel would read them
     StreamsUpdate   (a stream kept in several copies [S, T, E]) the update of all copies by a sublayer's result that
                     is still to be done; a norm that reads such a stream does it in its own pass over the rows
+    ScaledSum       scale * (a + b) still to be added: the two sublayers of a layer whose mixer and feed-forward read
+                    the same norm, and the layer's residual factor; a norm that says `adds_scaled_sum` takes it as delta
 
 What a part or a norm can do, it says with class attributes; a part without any gets and
 returns plain tensors, a norm without any does every sum and every normalisation in its own
@@ -81,6 +83,16 @@ class StreamsUpdate:
 
     def apply(self, x: torch.Tensor) -> None:
         self.lib.streams_update(x, self.mix, self.out_coef, self.y, self.scale)
+
+
+class ScaledSum:
+    """scale * (a + b) that is still to be added to the stream x [T, E]; b may be None."""
+
+    def __init__(self, a: torch.Tensor, b: Optional[torch.Tensor], scale: float):
+        self.a, self.b, self.scale = a, b, float(scale)
+
+    def parts(self):
+        return self.a, self.b, self.scale
 
 
 def normed_for(part, norm, x: torch.Tensor, pending, rows: Optional[torch.Tensor] = None):

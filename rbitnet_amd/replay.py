@@ -138,8 +138,9 @@ def main(argv: Optional[list] = None) -> int:
         # every live request holds at least one token and may leave most of its last page empty: room for that
         # many requests (256 at most), and a page more for each than their tokens alone would take
         slots = max(1, min(int(args.max_tokens), 256))
+        # no sequence is longer than the tokens that all may hold together: tables keyed by position need no more rows
         engine = Engine.load_path(args.model, dtype=args.dtype, max_tokens=int(args.max_tokens) + PAGE_SIZE * slots,
-                                  max_batch=slots)
+                                  max_batch=slots, max_seq_len=max(1, int(args.max_tokens)))
         replay(engine, sys.stdin, args.out)
     except RbitnetError as e:
         print(f"error: {e}", file=sys.stderr)
