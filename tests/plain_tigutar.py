@@ -241,3 +241,70 @@ class PlainTigutar:
                 layers_out.append(x.clone())
         x = layer_norm(x, self.w["final.norm"], self.w["final.norm.b"], eps)
         return x @ self.w["head"].T
+
+
+# ---------------------------------------------------------------- random weights for a configuration
+def random_tigutar_tensors(cfg: Dict, seed: int, decay_rank: int = 8) -> Dict[str, torch.Tensor]:
+    """Every tensor of a model of this configuration, float64 values that bfloat16 holds exactly.  Projections are
+    scaled so that scores, gates, decays and routers move with the input (a wrong mask, state or sink shows)."""
+    g = torch.Generator().manual_seed(seed)
+    e = cfg["width"]
+
+    def rnd(*shape, std=1.0, mean=0.0):
+        return (torch.randn(*shape, generator=g, dtype=F64) * std + mean).to(torch.bfloat16).to(F64)
+
+    def lin(n, k, gain=1.0):
+        return rnd(n, k, std=gain * k ** -0.5)
+
+    def softmax_tensors(p, prefix, gated):
+        out = {f"{prefix}q": lin(p["heads"] * p["dim"], e, 2.0), f"{prefix}o": lin(e, p["heads"] * p["vdim"])}
+        if p.get("kv_from") is None:
+            out[f"{prefix}k"] = lin(p["kv_heads"] * p["dim"], e, 2.0)
+            out[f"{prefix}v"] = lin(p["kv_heads"] * p["vdim"], e)
+        if gated:
+            out[f"{prefix}sink"] = rnd(p["heads"], std=1.5)
+            out[f"{prefix}g"] = lin(p["heads"], e, 2.0)
+        return out
+
+    t = {"embed": rnd(cfg["vocab"], e), "head": lin(cfg["vocab"], e), "final.norm": rnd(e, std=0.1, mean=1.0),
+         "final.norm.b": rnd(e, std=0.1)}
+    for i, layer in enumerate(cfg["layers"]):
+        pre, p = f"l{i}.", layer["mixer"]
+        t[pre + "norm1"], t[pre + "norm1.b"] = rnd(e, std=0.1, mean=1.0), rnd(e, std=0.1)
+        mx = pre + "mix."
+        if layer["type"] == "attention":
+            t.update(softmax_tensors(p, mx, True))
+        elif layer["type"] == "delta":
+            nqk, nv = p["kv_heads"] * p["dim"], p["heads"] * p["vdim"]
+            for name, n in (("q", nqk), ("k", nqk), ("v", nv)):
+                t[mx + name] = lin(n, e, 2.0)
+                t[mx + name + ".conv"] = rnd(n, p["conv"], std=0.6)
+            t[mx + "b"], t[mx + "a"] = lin(p["heads"], e, 2.0), lin(p["heads"], e, 2.0)
+            t[mx + "A_log"], t[mx + "dt_bias"] = rnd(p["heads"], std=0.5, mean=-1.0), rnd(p["heads"], std=0.5)
+            t[mx + "norm"] = rnd(p["vdim"], std=0.1, mean=1.0)
+            t[mx + "g"], t[mx + "o"] = lin(nv, e, 2.0), lin(e, nv)
+        else:
+            t.update(softmax_tensors(p["left"], mx + "left.", False))
+            r = p["right"]
+            rank = r.get("decay_rank", decay_rank)
+            nqk, nv = r["heads"] * r["dim"], r["heads"] * r["vdim"]
+            t[mx + "right.q"], t[mx + "right.k"], t[mx + "right.v"] = lin(nqk, e, 2.0), lin(nqk, e), lin(nv, e)
+            t[mx + "right.g"], t[mx + "right.o"] = lin(nv, e, 2.0), lin(e, nv)
+            t[mx + "right.norm"] = rnd(r["vdim"], std=0.1, mean=1.0)
+            t[mx + "right.a1"], t[mx + "right.a2"] = lin(rank, e, 2.0), lin(nqk, rank, 2.0)
+            t[mx + "right.a2.b"] = rnd(nqk, std=1.0, mean=2.0)
+            t[mx + "left.out"], t[mx + "right.out"] = rnd(e, std=0.1, mean=1.0), rnd(e, std=0.1, mean=1.0)
+        mlp = layer.get("mlp")
+        if mlp is None:
+            continue
+        fp = pre + "mlp."
+        if mlp["kind"] == "dense":
+            t[fp + "gate"], t[fp + "up"], t[fp + "down"] = lin(mlp["ff"], e, 2.0), lin(mlp["ff"], e), lin(e, mlp["ff"])
+        else:
+            ff = mlp["expert"]["ff"]
+            t[fp + "router"] = lin(mlp["router"]["experts"], e, 3.0)
+            for x in range(mlp["router"]["experts"]):
+                # large enough that the clamps of the gated unit are reached now and then
+                t[f"{fp}e{x}.gate"], t[f"{fp}e{x}.up"] = lin(ff, e, 3.0), lin(ff, e, 3.0)
+                t[f"{fp}e{x}.down"] = lin(e, ff)
+    return t
