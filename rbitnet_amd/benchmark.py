@@ -332,8 +332,37 @@ def bagonex_config(width: int, layers: int, heads: int, dim: int, ff: int, q_ran
             "canon": {"taps": 4}, "logit_softcap": 30.0, "layers": out}
 
 
-# size -> (the Bagonex configuration, the Llama shape of equal width, depth and feed-forward width beside it)
+def tigutar_config(width: int, layers: int, heads: int, kv_heads: int, ff: int, vocab: int, experts: int = 32, top: int = 4,
+                   window: int = 1024) -> dict:
+    """Groups of four parallel layers: attention with sinks and gates (every second one reads the keys and values of
+    the one four layers before it), the gated delta rule, and twice windowed attention (keys of 64, values of 128)
+    beside gated linear attention; dense feed-forwards alternate with routed experts whose `top` chosen ones are
+    together as wide as the dense one."""
+    soft = {"heads": heads, "kv_heads": kv_heads, "dim": 64, "vdim": 64, "rot": {"base": 500000.0, "dims": 64}, "scale": 0.125}
+    left = {"heads": heads // 2, "kv_heads": max(1, kv_heads // 2), "dim": 64, "vdim": 128, "rot": {"base": 1e6, "dims": 64},
+            "scale": 0.125, "mask": {"size": window}}
+    right = {"heads": max(1, heads // 4), "dim": 64, "vdim": 128, "tau": 16.0, "decay_rank": 64}
+    delta = {"heads": max(1, heads // 2), "kv_heads": max(1, heads // 4), "dim": 128, "vdim": 128, "conv": 4}
+    dense = {"kind": "dense", "ff": ff}
+    moe = {"kind": "moe", "expert": {"ff": ff // top, "limit": 7.0}, "router": {"experts": experts, "top": top}}
+    out = []
+    for i in range(layers):
+        kind = i % 4
+        if kind == 0:
+            mixer = dict(soft, kv_from=i - 4) if i % 8 == 4 else dict(soft)
+            out.append({"type": "attention", "mixer": mixer, "mlp": dense})
+        elif kind == 1:
+            out.append({"type": "delta", "mixer": dict(delta), "mlp": moe})
+        else:
+            out.append({"type": "parallel", "mixer": {"left": dict(left), "right": dict(right)}, "mlp": dense if kind == 2 else moe})
+    return {"architecture": "Tigutar", "vocab": vocab, "width": width, "residual_mult": 0.3, "norm": {"eps": 1e-5}, "layers": out}
+
+
+# size -> (the design's configuration, the Llama shape of equal width, depth and feed-forward width beside it)
 DESIGN_SIZES = {
+    "tigutar_w1024": (tigutar_config(1024, 12, 16, 4, 4096, 32000, experts=16), _other(1024, 4096, 16, 4, 64, 12, vocab=32000)),
+    "tigutar_w2048": (tigutar_config(2048, 16, 32, 8, 8192, 128256), _other(2048, 8192, 32, 8, 64, 16)),
+    "tigutar_w4096": (tigutar_config(4096, 8, 64, 16, 14336, 128256), dict(LLAMA3_8B, num_hidden_layers=8)),
     "w2048": (bagonex_config(2048, 16, 16, 128, 8192, 768, 128, 128256), _other(2048, 8192, 32, 8, 64, 16)),
     "w4096": (bagonex_config(4096, 8, 32, 128, 14336, 1536, 128, 128256), dict(LLAMA3_8B, num_hidden_layers=8)),
     "w1024": (bagonex_config(1024, 12, 8, 64, 4096, 384, 64, 32000, low_rank=64), _other(1024, 4096, 16, 4, 64, 12, vocab=32000)),
@@ -363,15 +392,16 @@ def _kernel_table(engine, run) -> dict:
 
 
 def design_run(size: str, dtype: str, batch: int, steps: int, warmup: int, prefill_tokens: int, prompt_len: int) -> dict:
-    """Prefill and decode throughput of a Bagonex model with random weights beside the Llama shape of equal size, and
-    where each spends its time, kernel by kernel."""
+    """Prefill and decode throughput of a model of another design with random weights beside the Llama shape of equal
+    size, and where each spends its time, kernel by kernel."""
     import numpy as np
     import torch
     from .engine import Engine
     out = {"size": size, "dtype": dtype, "batch": batch, "steps": steps, "prefill_tokens": prefill_tokens,
            "prompt_len": prompt_len}
-    for label, cfg in zip(("bagonex", "llama"), DESIGN_SIZES[size]):
+    for cfg in DESIGN_SIZES[size]:
         cfg = dict(cfg)
+        label = "llama" if "architectures" in cfg else str(cfg["architecture"]).lower()
         ctx_cap = prompt_len + steps + warmup + 64
         if "max_position_embeddings" in cfg:
             cfg["max_position_embeddings"] = max(cfg["max_position_embeddings"], prefill_tokens + 64, ctx_cap)
@@ -449,7 +479,7 @@ def main(argv=None) -> int:
                     help="no benchmark line: the named shape's decode products of 8 tokens beside a kernel that only "
                          "reads as many bytes")
     ap.add_argument("--design", default="", metavar="SIZE",
-                    help=f"no benchmark line: a Bagonex model of this size ({', '.join(sorted(DESIGN_SIZES))}) beside the Llama "
+                    help=f"no benchmark line: a Bagonex or Tigutar model of this size ({', '.join(sorted(DESIGN_SIZES))}) beside the Llama "
                          "shape of equal width, depth and feed-forward width: prefill and decode throughput, and the time per kernel")
     ap.add_argument("--tokens", default="1,8,64,512,2048", help="token counts of --planner-sweep")
     ap.add_argument("--sweep-detail", default=None, help="--planner-sweep: a file for every candidate's time")

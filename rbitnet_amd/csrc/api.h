@@ -226,16 +226,19 @@ int rb_pair_norm_mean(const float* a, const float* wa, const float* b, const flo
 // ---- a feed-forward of routed experts (routed.hip)
 // Router logits z [T, z_stride >= experts] -> the `top` experts with the largest sigmoid(z) per token (lowest index among
 // equals): sel, weight [T * top] (pair p = t * top + k), and the pairs sorted by expert in runs padded to 16 rows:
-// row_pair [max_rows] (-1: padding), tile_expert [max_rows / 16] (-1: past the end).  max_rows: a multiple of 16, at
-// least T * top rounded up to 16, plus 16 for every expert.
+// row_pair [max_rows] (-1: padding), tile_expert [2 * max_rows / 16]: the tiles' experts (-1: past the end), then the
+// tiles' positions in their experts' runs.  max_rows: a multiple of 16, at least T * top rounded up to 16, plus 16
+// for every expert.
 int rb_route_top(const float* z, long long z_stride, int n_experts, int top, int32_t* sel, float* weight, int32_t* row_pair,
                  int32_t* tile_expert, int max_rows, int n_tokens, void* stream);
 // For every pair p of token t: x = weight[p] h[t]; g = min(Wg x, limit), u = clamp(Wu x, -limit, limit);
 // out[p] = Wd (g sigmoid(alpha g) (u + 1)), the expert being the pair's.  w_gate, w_up [experts, ff, width] and w_down
-// [experts, width, ff] of dtype; y [max_rows, ff] of dtype is scratch; out [T * top, width] float32.
+// [experts, width, ff] of dtype; y [max_rows, ff + width] of dtype is scratch; out [T * top, width] float32.
+// w_layout 0: every expert's matrices as rows.  1 (bfloat16, width and ff multiples of 32): every expert's matrices
+// fragment-major, as rb_place_rows writes them; then the matrix cores run.
 int rb_routed_experts(const void* h, int dtype, const float* weight, int top, const int32_t* row_pair, const int32_t* tile_expert,
-                      int max_rows, const void* w_gate, const void* w_up, const void* w_down, void* y, float* out, int n_experts,
-                      int width, int ff, float limit, float alpha, void* stream);
+                      int max_rows, const void* w_gate, const void* w_up, const void* w_down, int w_layout, void* y, float* out,
+                      int n_experts, int width, int ff, float limit, float alpha, void* stream);
 // out[t] = sum over k of pairs[t * top + k], in the order of k.
 int rb_pairs_sum(const float* pairs, int top, float* out, int n_tokens, int width, void* stream);
 

@@ -172,7 +172,7 @@ class Kernels:
             "rb_head_gate": [_P, _I, _P, _L, _I, _I, _I, _P],
             "rb_pair_norm_mean": [_P, _P, _P, _P, _F, _P, _I, _I, _P],
             "rb_route_top": [_P, _L, _I, _I, _P, _P, _P, _P, _I, _I, _P],
-            "rb_routed_experts": [_P, _I, _P, _I, _P, _P, _I, _P, _P, _P, _P, _P, _I, _I, _I, _F, _F, _P],
+            "rb_routed_experts": [_P, _I, _P, _I, _P, _P, _I, _P, _P, _P, _I, _P, _P, _I, _I, _I, _F, _F, _P],
             "rb_pairs_sum": [_P, _I, _P, _I, _I, _P],
         }
         for name, args in sig.items():
@@ -760,28 +760,29 @@ class Kernels:
         _check(sel, "sel", torch.int32, (n * top,))
         _check(weight, "weight", torch.float32, (n * top,))
         _check(row_pair, "row_pair", torch.int32, (max_rows,))
-        _check(tile_expert, "tile_expert", torch.int32, (max_rows // 16,))
+        _check(tile_expert, "tile_expert", torch.int32, (2 * (max_rows // 16),))
         self._ok(self._lib.rb_route_top(_ptr(z), z.shape[1], n_experts, top, _ptr(sel), _ptr(weight), _ptr(row_pair),
                                         _ptr(tile_expert), max_rows, n, self._stream()))
 
     def routed_experts(self, h: torch.Tensor, weight: torch.Tensor, top: int, row_pair: torch.Tensor, tile_expert: torch.Tensor,
                        w_gate: torch.Tensor, w_up: torch.Tensor, w_down: torch.Tensor, y: torch.Tensor, out: torch.Tensor,
-                       limit: float, alpha: float) -> None:
+                       limit: float, alpha: float, w_frag: bool = False) -> None:
+        """w_frag: every expert's matrices are stored fragment-major (`place_rows(..., frag=True)` on each)."""
         n, width = h.shape
         n_experts, ff, _ = w_gate.shape
         max_rows = row_pair.shape[0]
         _check(h, "h")
         _check(weight, "weight", torch.float32, (n * top,))
         _check(row_pair, "row_pair", torch.int32)
-        _check(tile_expert, "tile_expert", torch.int32, (max_rows // 16,))
+        _check(tile_expert, "tile_expert", torch.int32, (2 * (max_rows // 16),))
         _check(w_gate, "w_gate", h.dtype, (n_experts, ff, width))
         _check(w_up, "w_up", h.dtype, (n_experts, ff, width))
         _check(w_down, "w_down", h.dtype, (n_experts, width, ff))
-        _check(y, "y", h.dtype, (max_rows, ff))
+        _check(y, "y", h.dtype, (max_rows, ff + width))
         _check(out, "out", torch.float32, (n * top, width))
         self._ok(self._lib.rb_routed_experts(_ptr(h), dtype_code(h.dtype), _ptr(weight), top, _ptr(row_pair), _ptr(tile_expert),
-                                             max_rows, _ptr(w_gate), _ptr(w_up), _ptr(w_down), _ptr(y), _ptr(out), n_experts, width,
-                                             ff, float(limit), float(alpha), self._stream()))
+                                             max_rows, _ptr(w_gate), _ptr(w_up), _ptr(w_down), int(bool(w_frag)), _ptr(y), _ptr(out),
+                                             n_experts, width, ff, float(limit), float(alpha), self._stream()))
 
     def pairs_sum(self, pairs: torch.Tensor, top: int, out: torch.Tensor) -> None:
         n, width = out.shape

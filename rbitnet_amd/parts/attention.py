@@ -64,8 +64,8 @@ class Attention(Part):
         self.head_dim = int(params["head_dim"])
         if self.n_heads <= 0 or self.n_kv <= 0 or self.n_heads % self.n_kv != 0:
             raise ConfigError(f"attention: {self.n_heads} heads cannot share {self.n_kv} kv heads")
-        if self.head_dim <= 0 or self.head_dim % 2 != 0 or self.head_dim > 256:
-            raise ConfigError(f"attention: head_dim {self.head_dim} not supported (even, at most 256)")
+        if self.head_dim <= 0 or self.head_dim > 512:
+            raise ConfigError(f"attention: head_dim {self.head_dim} not supported (at most 512)")
         self.value_dim = int(params.get("value_dim") or self.head_dim)
         if not 0 < self.value_dim <= 512:
             raise ConfigError(f"attention: value_dim {self.value_dim} not supported (1 to 512)")
@@ -84,6 +84,8 @@ class Attention(Part):
         self.rot = int(getattr(self.position, "head_dim", 0)) if getattr(self.position, "rotation_tables", None) else 0
         if self.rot > self.head_dim:
             raise ConfigError(f"attention: {self.rot} rotated numbers in a head of {self.head_dim}")
+        if self.rot % 2 != 0:
+            raise ConfigError(f"attention: a rotation pairs the numbers of a head, {self.rot} of them cannot be paired")
         self.pad = max(self.head_dim, self.value_dim)
         self.same_sizes = self.value_dim == self.head_dim and self.rot in (0, self.head_dim)
         self.w_gate = None

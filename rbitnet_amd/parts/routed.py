@@ -58,7 +58,17 @@ class RoutedExperts(Part):
         lib, allowed = self.env.lib, not getattr(self.env, "generic_only", False)
         r = tensors[self.names["router"]]
         self.w_router = pack_rows(lib, [(r, 0, None, None)], r.shape[0], r.shape[1], r.dtype, r.device, allowed)
-        stack = lambda what: torch.stack([tensors[self._name(i, what)] for i in range(self.n_experts)]).contiguous()
+        # all experts' matrices in one tensor each; for the matrix cores (bfloat16, sizes that are multiples of 32) every
+        # expert's matrix fragment-major, so that a wave's load is 1 KB in a row
+        self.frag = bool(allowed and r.dtype == torch.bfloat16 and self.hidden % 32 == 0 and self.ff % 32 == 0)
+
+        def stack(what: str) -> torch.Tensor:
+            first = tensors[self._name(0, what)]
+            out = torch.empty((self.n_experts,) + tuple(first.shape), dtype=first.dtype, device=first.device)
+            for i in range(self.n_experts):
+                lib.place_rows(tensors[self._name(i, what)].contiguous(), out[i], frag=self.frag)
+            return out
+
         self.w_gate, self.w_up, self.w_down = stack("gate"), stack("up"), stack("down")
 
     def forward(self, h: torch.Tensor, ctx=None, stream: Optional[torch.Tensor] = None, next_norm=None) -> torch.Tensor:
@@ -69,12 +79,12 @@ class RoutedExperts(Part):
         sel = torch.empty(pairs, dtype=torch.int32, device=dev)
         weight = torch.empty(pairs, dtype=torch.float32, device=dev)
         row_pair = torch.empty(max_rows, dtype=torch.int32, device=dev)
-        tile_expert = torch.empty(max_rows // 16, dtype=torch.int32, device=dev)
+        tile_expert = torch.empty(2 * (max_rows // 16), dtype=torch.int32, device=dev)      # experts, then positions in their runs
         lib.route_top(z, self.n_experts, self.top, sel, weight, row_pair, tile_expert)
-        y = torch.empty((max_rows, self.ff), dtype=h.dtype, device=dev)
+        y = torch.empty((max_rows, self.ff + self.hidden), dtype=h.dtype, device=dev)         # scratch: gated units, scaled inputs
         out = torch.empty((pairs, self.hidden), dtype=torch.float32, device=dev)
         lib.routed_experts(h, weight, self.top, row_pair, tile_expert, self.w_gate, self.w_up, self.w_down, y, out,
-                           self.limit, self.alpha)
+                           self.limit, self.alpha, w_frag=self.frag)
         if self.top == 1:
             return out
         total = torch.empty((t, self.hidden), dtype=torch.float32, device=dev)
