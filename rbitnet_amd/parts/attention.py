@@ -87,7 +87,7 @@ class Attention(Part):
         if self.rot % 2 != 0:
             raise ConfigError(f"attention: a rotation pairs the numbers of a head, {self.rot} of them cannot be paired")
         self.pad = max(self.head_dim, self.value_dim)
-        self.same_sizes = self.value_dim == self.head_dim and self.rot in (0, self.head_dim)
+        self.same_sizes = self.value_dim == self.head_dim and self.rot in (0, self.head_dim) and self.head_dim % 2 == 0
         self.w_gate = None
         self.sink: Optional[torch.Tensor] = None
         self.w_qkv: Optional[torch.Tensor] = None

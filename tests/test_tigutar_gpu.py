@@ -171,6 +171,9 @@ ATTENTIONS = [
     dict(heads=6, kv_heads=3, dim=64, vdim=128, rot={"base": 1e6, "dims": 32}, scale=0.1, mask={"size": 70}),  # padded to 128, window
     dict(heads=1, kv_heads=1, dim=6, vdim=5, rot={"base": 10.0, "dims": 0}, scale=1.0, mask={"size": 1}),      # no rotation, sees itself only
     dict(heads=2, kv_heads=1, dim=128, vdim=64, rot={"base": 300.0, "dims": 128}, scale=0.05, mask={"size": 64}),
+    dict(heads=2, kv_heads=1, dim=7, vdim=9, rot={"base": 20.0, "dims": 6}, scale=0.4, mask={"size": 129}),       # odd sizes
+    dict(heads=34, kv_heads=2, dim=64, vdim=64, rot={"base": 1e4, "dims": 64}, scale=0.125),                    # 17 heads on one
+    dict(heads=2, kv_heads=2, dim=5, vdim=5, rot={"base": 20.0, "dims": 0}, scale=0.5),
 ]
 
 
@@ -391,7 +394,15 @@ MODEL_C = {"architecture": "Tigutar", "vocab": 320, "width": 128, "residual_mult
     {"type": "attention", "mixer": _soft(4, 2, 64, 64, 64, 500000.0, 0.125, kv_from=0), "mlp": _dense(128)},
     {"type": "parallel", "mixer": {"left": _soft(2, 2, 128, 64, 32, 1e4, 0.09, mask={"size": 130}),
                                    "right": dict(heads=4, dim=16, vdim=16, tau=8.0, decay_rank=8)}, "mlp": _dense(256)}]}
-MODELS = {"A": (MODEL_A, 21), "B": (MODEL_B, 22), "C": (MODEL_C, 23)}
+# sizes off every grid: a width that is no multiple of 4, odd heads, seven experts of ten channels, one tap and nine
+MODEL_D = {"architecture": "Tigutar", "vocab": 37, "width": 50, "residual_mult": 0.7, "norm": {"eps": 1e-4}, "layers": [
+    {"type": "parallel", "mixer": {"left": _soft(3, 1, 10, 14, 6, 33.0, 0.3, mask={"size": 3}),
+                                   "right": dict(heads=3, dim=5, vdim=7, tau=3.0, decay_rank=3)}, "mlp": _moe(10, 0.8, 7, 3)},
+    {"type": "attention", "mixer": _soft(5, 5, 6, 6, 2, 7.0, 0.4), "mlp": None},
+    {"type": "delta", "mixer": dict(heads=6, kv_heads=2, dim=9, vdim=3, conv=9), "mlp": _dense(31)},
+    {"type": "attention", "mixer": _soft(5, 5, 6, 6, 2, 7.0, 0.6, kv_from=1), "mlp": _moe(9, 5.0, 2, 1)},
+    {"type": "delta", "mixer": dict(heads=1, kv_heads=1, dim=3, vdim=11, conv=1), "mlp": None}]}
+MODELS = {"A": (MODEL_A, 21), "B": (MODEL_B, 22), "C": (MODEL_C, 23), "D": (MODEL_D, 24)}
 _TMP = tempfile.TemporaryDirectory(prefix="tigutar_models_")
 _MADE = {}
 
@@ -457,7 +468,7 @@ def test_every_layer_of_a_model_against_the_plain_stream():
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["A", "B", "C"])
+@pytest.mark.parametrize("name", ["A", "B", "C", "D"])
 def test_model_whole_in_pieces_and_decoded(name, dtype):
     eng = _engine(name, dtype, max_tokens=64 * 12, max_batch=3)
     toks = _tokens(name, 200, 1)
@@ -473,7 +484,7 @@ def test_model_whole_in_pieces_and_decoded(name, dtype):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["A", "C"])
+@pytest.mark.parametrize("name", ["A", "C", "D"])
 def test_batches_of_unequal_requests_and_slots_used_again(name, dtype):
     """Four requests of 1 to 150 tokens start together and are decoded together, the short ones leaving early; then two
     new requests take the freed slots and pages.  Every request's logits are those it has alone."""
