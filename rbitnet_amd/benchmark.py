@@ -338,10 +338,10 @@ def tigutar_config(width: int, layers: int, heads: int, kv_heads: int, ff: int, 
     the one four layers before it), the gated delta rule, and twice windowed attention (keys of 64, values of 128)
     beside gated linear attention; dense feed-forwards alternate with routed experts whose `top` chosen ones are
     together as wide as the dense one."""
-    soft = {"heads": heads, "kv_heads": kv_heads, "dim": 64, "vdim": 64, "rot": {"base": 500000.0, "dims": 64}, "scale": 0.125}
-    left = {"heads": heads // 2, "kv_heads": max(1, kv_heads // 2), "dim": 64, "vdim": 128, "rot": {"base": 1e6, "dims": 64},
+    soft = {"heads": heads, "kv_heads": kv_heads, "dim": 64, "vdim": 64, "rot": {"base": 10000.0, "dims": 64}, "scale": 0.125}
+    left = {"heads": heads // 2, "kv_heads": max(1, kv_heads // 2), "dim": 64, "vdim": 128, "rot": {"base": 250000.0, "dims": 64},
             "scale": 0.125, "mask": {"size": window}}
-    right = {"heads": max(1, heads // 4), "dim": 64, "vdim": 128, "tau": 16.0, "decay_rank": 64}
+    right = {"heads": max(1, heads // 4), "dim": 64, "vdim": 128, "tau": 8.0, "decay_rank": 64}
     delta = {"heads": max(1, heads // 2), "kv_heads": max(1, heads // 4), "dim": 128, "vdim": 128, "conv": 4}
     dense = {"kind": "dense", "ff": ff}
     moe = {"kind": "moe", "expert": {"ff": ff // top, "limit": 7.0}, "router": {"experts": experts, "top": top}}
@@ -355,7 +355,7 @@ def tigutar_config(width: int, layers: int, heads: int, kv_heads: int, ff: int, 
             out.append({"type": "delta", "mixer": dict(delta), "mlp": moe})
         else:
             out.append({"type": "parallel", "mixer": {"left": dict(left), "right": dict(right)}, "mlp": dense if kind == 2 else moe})
-    return {"architecture": "Tigutar", "vocab": vocab, "width": width, "residual_mult": 0.3, "norm": {"eps": 1e-5}, "layers": out}
+    return {"architecture": "Tigutar", "vocab": vocab, "width": width, "residual_mult": 0.5, "norm": {"eps": 1e-5}, "layers": out}
 
 
 # size -> (the design's configuration, the Llama shape of equal width, depth and feed-forward width beside it)

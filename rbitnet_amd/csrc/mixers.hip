@@ -55,6 +55,64 @@ __global__ void rope_store_kernel(const float* __restrict__ qkv, size_t row_widt
   }
 }
 
+// The same with four numbers a thread (16-byte loads, 8- or 16-byte stores), for sizes that are multiples of 4 and a
+// rotated part that is a multiple of 8: a group of four lies wholly in the first half of the rotated part, in its
+// second half, behind it, or in the padding.
+__device__ __forceinline__ void store4(float* p, float a, float b, float c, float d) { *reinterpret_cast<float4*>(p) = make_float4(a, b, c, d); }
+__device__ __forceinline__ void store4(bf16_t* p, float a, float b, float c, float d) {
+  *reinterpret_cast<uint2*>(p) = make_uint2(pack_bf16x2(a, b), pack_bf16x2(c, d));
+}
+template <typename TC>
+__global__ void rope_store_vec_kernel(const float* __restrict__ qkv, size_t row_width, const float* __restrict__ cos_t,
+                                      const float* __restrict__ sin_t, int rot, TC* __restrict__ q_out, TC* __restrict__ k_pages,
+                                      TC* __restrict__ v_pages, const int32_t* __restrict__ tok_pos,
+                                      const int32_t* __restrict__ tok_seq, const int32_t* __restrict__ block_table, int bt_stride,
+                                      int n_heads, int n_kv, int dim, int vdim, int pad) {
+  const int t = blockIdx.x;
+  const int pos = tok_pos[t];
+  const int half = rot / 2;
+  const float* src = qkv + (size_t)t * row_width;
+  const float* cr = cos_t + (size_t)pos * half;
+  const float* sr = sin_t + (size_t)pos * half;
+  size_t page_base = 0;
+  if (k_pages) {
+    const int page = block_table[(size_t)tok_seq[t] * bt_stride + pos / RB_PAGE];
+    page_base = ((size_t)page * n_kv) * RB_PAGE * pad + (size_t)(pos % RB_PAGE) * pad;
+  }
+  const int n_rot_heads = n_heads + (k_pages ? n_kv : 0);
+  const int quads = pad / 4;
+  for (int idx = threadIdx.x; idx < n_rot_heads * quads; idx += blockDim.x) {
+    const int h = idx / quads, d = 4 * (idx - h * quads);
+    const float* hp = src + (size_t)h * dim;
+    float4 y = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (d < rot) {
+      const bool first = d < half;
+      const int i = first ? d : d - half;                       // the pairs' index
+      const float4 a = *reinterpret_cast<const float4*>(hp + i), b = *reinterpret_cast<const float4*>(hp + i + half);
+      const float4 c = *reinterpret_cast<const float4*>(cr + i), sn = *reinterpret_cast<const float4*>(sr + i);
+      float y0[4], y1[4];
+      rotate_pair(a.x, b.x, c.x, sn.x, y0[0], y1[0]);
+      rotate_pair(a.y, b.y, c.y, sn.y, y0[1], y1[1]);
+      rotate_pair(a.z, b.z, c.z, sn.z, y0[2], y1[2]);
+      rotate_pair(a.w, b.w, c.w, sn.w, y0[3], y1[3]);
+      y = first ? make_float4(y0[0], y0[1], y0[2], y0[3]) : make_float4(y1[0], y1[1], y1[2], y1[3]);
+    } else if (d < dim) {
+      y = *reinterpret_cast<const float4*>(hp + d);
+    }
+    TC* dst = h < n_heads ? q_out + ((size_t)t * n_heads + h) * pad
+                          : k_pages + page_base + (size_t)(h - n_heads) * RB_PAGE * pad;
+    store4(dst + d, y.x, y.y, y.z, y.w);
+  }
+  if (v_pages) {
+    const float* vsrc = src + (size_t)(n_heads + n_kv) * dim;
+    for (int idx = threadIdx.x; idx < n_kv * quads; idx += blockDim.x) {
+      const int h = idx / quads, d = 4 * (idx - h * quads);
+      const float4 v = d < vdim ? *reinterpret_cast<const float4*>(vsrc + (size_t)h * vdim + d) : make_float4(0.f, 0.f, 0.f, 0.f);
+      store4(v_pages + page_base + (size_t)h * RB_PAGE * pad + d, v.x, v.y, v.z, v.w);
+    }
+  }
+}
+
 extern "C" int rb_rope_store(const float* qkv, long long row_width, const float* cos, const float* sin, int rot, void* q_out,
                              void* k_pages, void* v_pages, int cache_dtype, const int32_t* tok_pos, const int32_t* tok_seq,
                              const int32_t* block_table, int bt_stride, int n_tokens, int n_heads, int n_kv_heads, int dim,
@@ -70,7 +128,18 @@ extern "C" int rb_rope_store(const float* qkv, long long row_width, const float*
   RB_REQUIRE(row_width >= need, "rb_rope_store: rows of %lld numbers, %lld needed", row_width, need);
   if (n_tokens == 0) return 0;
   hipStream_t s = (hipStream_t)stream;
-  if (cache_dtype == RB_F32)
+  auto aligned = [](const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; };
+  const bool vec = dim % 4 == 0 && vdim % 4 == 0 && pad % 4 == 0 && rot % 8 == 0 && row_width % 4 == 0 && aligned(qkv) &&
+                   aligned(cos) && aligned(sin) && aligned(q_out) && aligned(k_pages) && aligned(v_pages);
+  if (vec && cache_dtype == RB_F32)
+    rope_store_vec_kernel<float><<<n_tokens, 256, 0, s>>>(qkv, (size_t)row_width, cos, sin, rot, (float*)q_out, (float*)k_pages,
+                                                          (float*)v_pages, tok_pos, tok_seq, block_table, bt_stride, n_heads,
+                                                          n_kv_heads, dim, vdim, pad);
+  else if (vec && cache_dtype == RB_BF16)
+    rope_store_vec_kernel<bf16_t><<<n_tokens, 256, 0, s>>>(qkv, (size_t)row_width, cos, sin, rot, (bf16_t*)q_out, (bf16_t*)k_pages,
+                                                           (bf16_t*)v_pages, tok_pos, tok_seq, block_table, bt_stride, n_heads,
+                                                           n_kv_heads, dim, vdim, pad);
+  else if (cache_dtype == RB_F32)
     rope_store_kernel<float><<<n_tokens, 256, 0, s>>>(qkv, (size_t)row_width, cos, sin, rot, (float*)q_out, (float*)k_pages,
                                                       (float*)v_pages, tok_pos, tok_seq, block_table, bt_stride, n_heads,
                                                       n_kv_heads, dim, vdim, pad);
@@ -98,15 +167,52 @@ __global__ void head_gate_kernel(TC* __restrict__ x, const float* __restrict__ g
   }
 }
 
+// The same with 16 bytes a lane, for head sizes that are multiples of 8: a group of values lies within one head.
+template <typename TC>
+__global__ void head_gate_vec_kernel(TC* __restrict__ x, const float* __restrict__ gate, size_t gate_stride, int n_heads, int d,
+                                     size_t n_groups) {
+  constexpr int E = 16 / sizeof(TC);
+  for (size_t gi = (size_t)blockIdx.x * blockDim.x + threadIdx.x; gi < n_groups; gi += (size_t)gridDim.x * blockDim.x) {
+    const size_t e = gi * E;
+    const size_t th = e / d;
+    const size_t t = th / n_heads;
+    const int h = (int)(th - t * n_heads);
+    const float g = 1.0f / (1.0f + expf(-gate[t * gate_stride + h]));
+    uint4 raw = *reinterpret_cast<const uint4*>(x + e);
+    if (sizeof(TC) == 4) {
+      float4 v = *reinterpret_cast<float4*>(&raw);
+      v = make_float4(v.x * g, v.y * g, v.z * g, v.w * g);
+      *reinterpret_cast<float4*>(x + e) = v;
+    } else {
+      raw = make_uint4(pack_bf16x2(bf16_bits_to_f32(raw.x & 0xffffu) * g, bf16_bits_to_f32(raw.x >> 16) * g),
+                       pack_bf16x2(bf16_bits_to_f32(raw.y & 0xffffu) * g, bf16_bits_to_f32(raw.y >> 16) * g),
+                       pack_bf16x2(bf16_bits_to_f32(raw.z & 0xffffu) * g, bf16_bits_to_f32(raw.z >> 16) * g),
+                       pack_bf16x2(bf16_bits_to_f32(raw.w & 0xffffu) * g, bf16_bits_to_f32(raw.w >> 16) * g));
+      *reinterpret_cast<uint4*>(x + e) = raw;
+    }
+  }
+}
+
 extern "C" int rb_head_gate(void* x, int dtype, const float* gate, long long gate_stride, int n_tokens, int n_heads, int head_dim,
                             void* stream) {
   RB_RECORDED(rb_head_gate(x, dtype, gate, gate_stride, n_tokens, n_heads, head_dim, stream));
   RB_REQUIRE(n_tokens >= 0 && n_heads > 0 && head_dim > 0 && gate_stride >= n_heads, "rb_head_gate: bad sizes");
   if (n_tokens == 0) return 0;
   const size_t n = (size_t)n_tokens * n_heads * head_dim;
+  hipStream_t s = (hipStream_t)stream;
+  if (head_dim % 8 == 0 && (reinterpret_cast<uintptr_t>(x) & 15) == 0 && (dtype == RB_F32 || dtype == RB_BF16)) {
+    const size_t groups = n / (dtype == RB_F32 ? 4 : 8);
+    const size_t vb = (groups + 255) / 256;
+    const int vgrid = (int)(vb < 65535 ? vb : 65535);
+    if (dtype == RB_F32)
+      head_gate_vec_kernel<float><<<vgrid, 256, 0, s>>>((float*)x, gate, (size_t)gate_stride, n_heads, head_dim, groups);
+    else
+      head_gate_vec_kernel<bf16_t><<<vgrid, 256, 0, s>>>((bf16_t*)x, gate, (size_t)gate_stride, n_heads, head_dim, groups);
+    RB_LAUNCH_CHECK();
+    return 0;
+  }
   const size_t blocks = (n + 255) / 256;
   const int grid = (int)(blocks < 65535 ? blocks : 65535);
-  hipStream_t s = (hipStream_t)stream;
   if (dtype == RB_F32)
     head_gate_kernel<float><<<grid, 256, 0, s>>>((float*)x, gate, (size_t)gate_stride, n_heads, head_dim, n);
   else if (dtype == RB_BF16)
@@ -136,11 +242,52 @@ __global__ void pair_norm_mean_kernel(const float* __restrict__ a, const float* 
     out[r * width + j] = 0.5f * (ar[j] * fa * wa[j] + br[j] * fb * wb[j]);
 }
 
+// The same with 16-byte accesses for widths that are multiples of 4, the rows kept in registers between the two passes
+// when 1024 threads hold them (widths up to 4096), else read again.
+__global__ __launch_bounds__(1024) void pair_norm_mean_vec_kernel(const float* __restrict__ a, const float* __restrict__ wa,
+                                                                  const float* __restrict__ b, const float* __restrict__ wb, float eps,
+                                                                  float* __restrict__ out, int width) {
+  __shared__ float scratch[16];
+  const size_t r = blockIdx.x;
+  const float* ar = a + r * width;
+  const float* br = b + r * width;
+  const int j0 = 4 * threadIdx.x;
+  float4 va = make_float4(0.f, 0.f, 0.f, 0.f), vb = va;
+  float sa = 0.f, sb = 0.f;
+  for (int j = j0; j < width; j += 4 * blockDim.x) {
+    const float4 x = *reinterpret_cast<const float4*>(ar + j), y = *reinterpret_cast<const float4*>(br + j);
+    if (j == j0) {
+      va = x;
+      vb = y;
+    }
+    sa += (x.x * x.x + x.y * x.y) + (x.z * x.z + x.w * x.w);
+    sb += (y.x * y.x + y.y * y.y) + (y.z * y.z + y.w * y.w);
+  }
+  const float fa = 1.0f / sqrtf(block_sum(sa, scratch) / (float)width + eps);
+  const float fb = 1.0f / sqrtf(block_sum(sb, scratch) / (float)width + eps);
+  for (int j = j0; j < width; j += 4 * blockDim.x) {
+    const float4 x = j == j0 ? va : *reinterpret_cast<const float4*>(ar + j);
+    const float4 y = j == j0 ? vb : *reinterpret_cast<const float4*>(br + j);
+    const float4 p = *reinterpret_cast<const float4*>(wa + j), q = *reinterpret_cast<const float4*>(wb + j);
+    *reinterpret_cast<float4*>(out + r * width + j) =
+        make_float4(0.5f * (x.x * fa * p.x + y.x * fb * q.x), 0.5f * (x.y * fa * p.y + y.y * fb * q.y),
+                    0.5f * (x.z * fa * p.z + y.z * fb * q.z), 0.5f * (x.w * fa * p.w + y.w * fb * q.w));
+  }
+}
+
 extern "C" int rb_pair_norm_mean(const float* a, const float* wa, const float* b, const float* wb, float eps, float* out,
                                  int n_tokens, int width, void* stream) {
   RB_RECORDED(rb_pair_norm_mean(a, wa, b, wb, eps, out, n_tokens, width, stream));
   RB_REQUIRE(n_tokens >= 0 && width > 0, "rb_pair_norm_mean: bad sizes %d x %d", n_tokens, width);
   if (n_tokens == 0) return 0;
+  auto aligned = [](const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; };
+  if (width % 4 == 0 && aligned(a) && aligned(b) && aligned(wa) && aligned(wb) && aligned(out)) {
+    int threads = ((width / 4 + RB_WAVE - 1) / RB_WAVE) * RB_WAVE;
+    if (threads > 1024) threads = 1024;
+    pair_norm_mean_vec_kernel<<<n_tokens, threads, 0, (hipStream_t)stream>>>(a, wa, b, wb, eps, out, width);
+    RB_LAUNCH_CHECK();
+    return 0;
+  }
   const int threads = width >= 1024 ? 1024 : (width >= 256 ? 256 : 64);
   pair_norm_mean_kernel<<<n_tokens, threads, 0, (hipStream_t)stream>>>(a, wa, b, wb, eps, out, width);
   RB_LAUNCH_CHECK();

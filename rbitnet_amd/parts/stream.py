@@ -6,7 +6,7 @@ does it but by whoever can do it without a pass of its own over memory: the norm
 (its kernel adds `pending` to x before it normalises), or, in a step of few tokens, the
 part's last product (which adds its float32 sums to x in its epilogue and leaves the rows
 prepared for the norm that follows, `GainedRows`).  What a sublayer has not yet added is
-`pending`, and it takes one of four forms:
+`pending`, and it takes one of these forms:
 
     None            nothing: the stream holds the sum already
     tensor [T, E]   a float32 term still to be added
