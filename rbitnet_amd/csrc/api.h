@@ -140,6 +140,11 @@ int rb_attention_decode_bf16_sinks(const void* q, const void* k_pages, const voi
                                    const int32_t* tok_pos, const int32_t* block_table, int bt_stride, int n_seqs,
                                    int n_heads, int n_kv_heads, int head_dim, float scale, int window, int n_splits,
                                    float* workspace, const float* sinks, void* stream);
+int rb_attention_decode_fused_bf16_sinks(const float* qkv, int qkv_terms, long long qkv_term_stride, const float* cos,
+                                         const float* sin, int style, void* k_pages, void* v_pages, void* out,
+                                         const int32_t* tok_pos, const int32_t* block_table, int bt_stride, int n_seqs,
+                                         int n_heads, int n_kv_heads, int head_dim, float scale, int window, int n_splits,
+                                         float* workspace, const float* sinks, void* stream);
 
 // ---- a residual stream in several copies, layer norm, xIELU, the cap of logits (streams.hip)
 // x [S, T, E] float32, stream_stride floats from one copy to the next.

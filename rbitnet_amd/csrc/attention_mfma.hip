@@ -1139,15 +1139,26 @@ extern "C" int rb_attention_decode_fused_bf16(const float* qkv, int qkv_terms, l
                                               const int32_t* block_table, int bt_stride, int n_seqs, int n_heads,
                                               int n_kv_heads, int head_dim, float scale, int window, int n_splits,
                                               float* workspace, void* stream) {
-  RB_RECORDED(rb_attention_decode_fused_bf16(qkv, qkv_terms, qkv_term_stride, cos, sin, style, k_pages, v_pages, out, tok_pos,
-                                             block_table, bt_stride, n_seqs, n_heads, n_kv_heads, head_dim, scale, window,
-                                             n_splits, workspace, stream));
+  return rb_attention_decode_fused_bf16_sinks(qkv, qkv_terms, qkv_term_stride, cos, sin, style, k_pages, v_pages, out, tok_pos,
+                                              block_table, bt_stride, n_seqs, n_heads, n_kv_heads, head_dim, scale, window,
+                                              n_splits, workspace, nullptr, stream);
+}
+
+extern "C" int rb_attention_decode_fused_bf16_sinks(const float* qkv, int qkv_terms, long long qkv_term_stride,
+                                                    const float* cos, const float* sin, int style,
+                                                    void* k_pages, void* v_pages, void* out, const int32_t* tok_pos,
+                                                    const int32_t* block_table, int bt_stride, int n_seqs, int n_heads,
+                                                    int n_kv_heads, int head_dim, float scale, int window, int n_splits,
+                                                    float* workspace, const float* sinks, void* stream) {
+  RB_RECORDED(rb_attention_decode_fused_bf16_sinks(qkv, qkv_terms, qkv_term_stride, cos, sin, style, k_pages, v_pages, out,
+                                                   tok_pos, block_table, bt_stride, n_seqs, n_heads, n_kv_heads, head_dim, scale,
+                                                   window, n_splits, workspace, sinks, stream));
   RB_REQUIRE((cos == nullptr) == (sin == nullptr), "rb_attention_decode_fused_bf16: cos and sin tables go together");
   RB_REQUIRE(style == 0 || style == 1, "rb_attention_decode_fused_bf16: unknown pairing style %d", style);
   RB_REQUIRE(qkv_terms >= 1 && qkv_term_stride >= 0, "rb_attention_decode_fused_bf16: %d terms, %lld apart", qkv_terms,
              qkv_term_stride);
   DecodeArgs a = {qkv, nullptr, cos, sin, style, (bf16_t*)k_pages, (bf16_t*)v_pages, (bf16_t*)out,
                   tok_pos, block_table, bt_stride, n_seqs, n_heads, n_kv_heads, scale * LOG2E, window, n_splits,
-                  workspace, qkv_terms, (size_t)qkv_term_stride, nullptr};
+                  workspace, qkv_terms, (size_t)qkv_term_stride, sinks};
   return dispatch_decode<true>(a, head_dim, (hipStream_t)stream, "rb_attention_decode_fused_bf16");
 }

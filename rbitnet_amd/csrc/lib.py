@@ -144,6 +144,8 @@ class Kernels:
             "rb_attention_decode_bf16": [_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _F, _I, _I, _P, _P],
             "rb_attention_decode_fused_bf16": [_P, _I, ctypes.c_longlong, _P, _P, _I, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _F, _I, _I,
                                                _P, _P],
+            "rb_attention_decode_fused_bf16_sinks": [_P, _I, ctypes.c_longlong, _P, _P, _I, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I,
+                                                     _F, _I, _I, _P, _P, _P],
             "rb_sample": [_P, _I, _I, _P, _P, _P, _P, _P],
             "rb_fill_normal": [_P, _I, ctypes.c_longlong, ctypes.c_ulonglong, ctypes.c_double, ctypes.c_double, _P],
             "rb_place_rows": [_P, _I, _P, _I, _I] + [ctypes.c_longlong] * 6 + [_P],
@@ -411,7 +413,7 @@ class Kernels:
                                                           _ptr(workspace), _ptr(sinks), self._stream()))
 
     def attention_decode_fused_bf16(self, qkv, cos, sin, style, k_pages, v_pages, out, tok_pos, block_table,
-                                    n_heads, n_kv, head_dim, scale, window, n_splits, workspace) -> None:
+                                    n_heads, n_kv, head_dim, scale, window, n_splits, workspace, sinks=None) -> None:
         n, n_terms, term_stride = _terms(qkv, (n_heads + 2 * n_kv) * head_dim)
         if cos is not None:
             _check(cos, "cos", torch.float32)
@@ -428,11 +430,13 @@ class Kernels:
         _check(workspace, "workspace", torch.float32)
         if workspace.numel() < n * n_heads * n_splits * (head_dim + 2):
             raise KernelError("decode attention workspace too small")
-        self._ok(self._lib.rb_attention_decode_fused_bf16(
+        if sinks is not None:
+            _check(sinks, "sinks", torch.float32, (n_heads,))
+        self._ok(self._lib.rb_attention_decode_fused_bf16_sinks(
             _ptr(qkv), n_terms, term_stride, _ptr(cos), _ptr(sin), int(style), _ptr(k_pages), _ptr(v_pages), _ptr(out),
             _ptr(tok_pos),
             _ptr(block_table), block_table.shape[1], n, n_heads, n_kv, head_dim, float(scale), int(window or 0),
-            int(n_splits), _ptr(workspace), self._stream()))
+            int(n_splits), _ptr(workspace), _ptr(sinks), self._stream()))
 
     def sample(self, logits: torch.Tensor, temperature: Optional[torch.Tensor], u: Optional[torch.Tensor],
                tokens: torch.Tensor, workspace: Optional[torch.Tensor] = None) -> None:

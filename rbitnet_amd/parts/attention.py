@@ -167,12 +167,12 @@ class Attention(Part):
                 and not getattr(self.env, "generic_only", False))
         decode = fast and ctx.max_q_len == 1 and (hq // hk) in _DECODE_GROUPS
         tables = getattr(self.position, "rotation_tables", None)
-        if decode and owns and tables is not None and self.same_sizes and not self.has_sink:
+        if decode and owns and tables is not None and self.same_sizes:
             # one kernel: rotation, cache write, attention over the pages
             cos, sin, style = tables()
             n_splits, workspace = ctx.decode_workspace(hq, d, hk)
             lib.attention_decode_fused_bf16(qkv, cos, sin, style, view.k_pages, view.v_pages, attn, ctx.tok_pos, bt,
-                                            hq, hk, d, self.scale, window, n_splits, workspace)
+                                            hq, hk, d, self.scale, window, n_splits, workspace, sinks=self.sink)
             return self._gate_and_project(attn, h, stream, next_norm)
         q = torch.empty((t, hq, d), dtype=self.env.dtype, device=h.device)
         if self.same_sizes:
